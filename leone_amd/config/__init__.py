@@ -2,3 +2,4 @@ from .base import ConfigError, UnsupportedArchitecture, architecture_name, read_
 from .qwen3 import Qwen3Config
 from .pamevik import PamevikConfig
 from .zukinex import ZukinexConfig
+from .fosulix import FosulixConfig

@@ -163,10 +163,21 @@ inline int ceil_div(long a, long b) { return static_cast<int>((a + b - 1) / b); 
 
 // The activation of the gate of a gated feed-forward: 0 silu(g) = g / (1 + exp(-g)); 1 the tanh form of gelu,
 // 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).
-enum GateAct : int { kGateSilu = 0, kGateGeluTanh = 1 };
+// 2 a gate and an up value held to a limit: g = min(g, limit), u = clamp(u, -limit, limit), g sigmoid(1.702 g) (u + 1).
+enum GateAct : int { kGateSilu = 0, kGateGeluTanh = 1, kGateClampedSwish = 2 };
 __device__ inline float gate_act(float g, int act) {
     if (act == kGateGeluTanh) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
     return g / (1.0f + expf(-g));
+}
+
+// act(gate) * up of a gated feed-forward; `limit` belongs to kGateClampedSwish alone.
+__device__ inline float glu_value(float g, float u, int act, float limit) {
+    if (act == kGateClampedSwish) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    }
+    return gate_act(g, act) * u;
 }
 
 }  // namespace leone

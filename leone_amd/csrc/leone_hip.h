@@ -283,9 +283,12 @@ int leone_attention_prefill_kept(const void* q, void* out, const void* k_pool, c
                                  int kv_heads, int head_dim, int page_tokens, float scale, int window, float* part_acc,
                                  float* part_ml, int splits, int keep_first, hipStream_t stream);
 // Router: chosen int32 [rows, top], weight float32 [rows, top] from logits float32 [rows, total] (see routed.hip).
+// score: 0 softmax over the outputs, 1 a sigmoid of each; group_best: how many of a group's best choice scores are summed
+// into the group's score; renorm: the winners' scores over their sum (1) or as they are (0); weight_scale multiplies them.
 int leone_route_max_outputs();
 int leone_route_topk(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight,
-                     int rows, int total, int top, int group_count, int group_keep, hipStream_t stream);
+                     int rows, int total, int top, int group_count, int group_keep, int score, int group_best, int renorm,
+                     float weight_scale, hipStream_t stream);
 // Pairs (row, place) of the experts below `experts` gathered in tiles of `tile` pairs of one expert (leone_moe_tile_pairs(),
 // 16, 64 or 128): tile_expert int32 [max_tiles] (-1: unused), tile_pairs int32 [max_tiles, tile] (-1: empty);
 // max_tiles >= min(pairs, pairs / tile + experts).
@@ -294,13 +297,39 @@ int leone_moe_tile_pairs();
 // so many of the experts are taken by every row with weight 1 (chosen and weight are [rows, top + always] then).
 int leone_route_plan(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight, int rows,
                      int total, int top, int group_count, int group_keep, int experts, int* tile_expert, int* tile_pairs,
-                     int max_tiles, int tile, int always, hipStream_t stream);
+                     int max_tiles, int tile, int always, int score, int group_best, int renorm, float weight_scale,
+                     hipStream_t stream);
 int leone_moe_plan(const int* chosen, int pairs, int experts, int* tile_expert, int* tile_pairs, int max_tiles, int tile,
                    hipStream_t stream);
 // tile: leone_moe_tile_pairs() (any type and size), or 16, 64 or 128 (matrix cores: bfloat16, n and k multiples of 8).
 int leone_moe_product(const void* x, const void* w, void* y, const float* pair_weight, int dtype, int gated,
                       const int* tile_expert, const int* tile_pairs, int max_tiles, int tile, int top, int n, int k, int act,
-                      hipStream_t stream);
+                      float limit, hipStream_t stream);
 int leone_moe_combine(const float* pair_out, const int* chosen, const float* weight, const void* x, int dtype,
                       const float* extra, float* out, int rows, int top, int experts, int hidden, hipStream_t stream);
+// A matrix memory whose forget gate per head and key channel also says what is written (see gated_scan.hip).
+int leone_gated_scan(const float* proj, long stride, int q_off, int f_off, int v_off, const void* f_bias, const void* lower,
+                     int vec_dtype, int q_silu, int no_input, int accumulate, const int* segments, int n_segments,
+                     const float* state_in, long in_stride, float* state_out, long out_stride, float* gate_product, float* out,
+                     int heads, int dim, int vdim, hipStream_t stream);
+int leone_gated_chain(const int* links, int n_links, float* work, long work_stride, const float* product, float* state,
+                      long slot_stride, int heads, int dim, int vdim, int write_state, hipStream_t stream);
+// Attention through a latent that all heads share (see latent.hip).
+int leone_latent_max_width();
+int leone_latent_prepare(const float* proj, long stride, int rows, int q_off, int q_rank, const void* q_gain, void* q_out,
+                         int kv_off, int rank, int rot, const void* kv_gain, int gain_dtype, float eps, const float* cos_table,
+                         const float* sin_table, int rot_half, int table_positions, const int* positions, const int* row_entry,
+                         const int* block_table, int max_blocks, int page_tokens, void* pool, int dtype, hipStream_t stream);
+int leone_head_product(const float* x, long x_row_stride, long x_head_stride, const void* w, int w_dtype, void* y, int y_dtype,
+                       long y_row_stride, long y_head_stride, int rows, int heads, int inner, int outer, int tail,
+                       const float* cos_table, const float* sin_table, int rot_half, int table_positions, const int* positions,
+                       hipStream_t stream);
+int leone_latent_attention(const float* q, float* out, const void* pool, int dtype, const int* positions, const int* row_entry,
+                           const int* block_table, int max_blocks, int rows, int heads, int rank, int rot, int page_tokens,
+                           float scale, int window, hipStream_t stream);
+// Residual sums with a factor; the stream as a weighted sum of every earlier layer's result (see depth.hip).
+int leone_residual_norm(float* x, const float* delta, int planes, long plane, float scale, const void* gain, int gain_dtype,
+                        float eps, void* y, int y_dtype, const int* rows, int n_rows, int hidden, hipStream_t stream);
+int leone_depth_mix(float* x, const float* delta, int planes, long plane, float scale, float* history, long slot_stride,
+                    int count, const void* weight, int weight_dtype, long total, hipStream_t stream);
 }

@@ -45,10 +45,18 @@ __device__ inline void wave_best(float& v, int& at) {
 }
 
 // One wave a row; a lane holds kSlots router outputs (kSlots * 64 >= total).
+// How a router scores and weighs: `score` 0 softmax over all outputs, 1 a sigmoid of each; `group_best` how many of a
+// group's best choice scores make the group's score (their sum; 1: the best alone); `renorm` 1: the winners' scores over
+// their sum, 0: the scores themselves; `scale` multiplies the weights either way.
+struct RouteRule {
+    int score, group_best, renorm;
+    float scale;
+};
+
 template <int kSlots>
 __device__ inline void route_row(int row, int lane, const float* __restrict__ logits, const AnyVec& correction,
                                  int* __restrict__ chosen, float* __restrict__ weight, int total, int top, int group_count,
-                                 int group_keep, int shift_from = 0x7fffffff, int always = 0) {
+                                 int group_keep, const RouteRule rule, int shift_from = 0x7fffffff, int always = 0) {
     // `always` experts that every row takes with weight 1 stand behind the routed ones in the matrices (indices
     // shift_from .. shift_from + always - 1): a row's places are its `top` choices and then these; a chosen router
     // output from shift_from on (one that hands the row on) is numbered behind them.
@@ -68,10 +76,11 @@ __device__ inline void route_row(int row, int lane, const float* __restrict__ lo
 #pragma unroll
     for (int i = 0; i < kSlots; ++i) {
         const int e = lane + i * kWave;
-        s[i] = e < total ? expf(s[i] - top_z) : 0.f;
+        if (rule.score == 1) s[i] = e < total ? 1.0f / (1.0f + expf(-s[i])) : 0.f;
+        else s[i] = e < total ? expf(s[i] - top_z) : 0.f;
         sum += s[i];
     }
-    sum = wave_sum(sum);
+    sum = rule.score == 1 ? 1.0f : wave_sum(sum);
 #pragma unroll
     for (int i = 0; i < kSlots; ++i) {
         const int e = lane + i * kWave;
@@ -93,13 +102,27 @@ __device__ inline void route_row(int row, int lane, const float* __restrict__ lo
             mine_taken[i] = lane + i * kWave >= group_count;
         }
         for (int g = 0; g < group_count; ++g) {
-            float best = -INFINITY;
+            float best = 0.f;
+            int used[kSlots];                              // the group's outputs already counted into its score
 #pragma unroll
-            for (int i = 0; i < kSlots; ++i) {
-                const int e = lane + i * kWave;
-                if (e < total && group_of[i] == g) best = fmaxf(best, choice[i]);
+            for (int i = 0; i < kSlots; ++i) used[i] = 0;
+            for (int n = 0; n < rule.group_best && n < size; ++n) {
+                float v = -INFINITY;
+                int at = 0x7fffffff;
+#pragma unroll
+                for (int i = 0; i < kSlots; ++i) {
+                    const int e = lane + i * kWave;
+                    if (e < total && group_of[i] == g && !used[i] && (at == 0x7fffffff || choice[i] > v)) {
+                        v = choice[i];
+                        at = e;
+                    }
+                }
+                wave_best(v, at);
+#pragma unroll
+                for (int i = 0; i < kSlots; ++i)
+                    if (lane + i * kWave == at) used[i] = 1;
+                best = n == 0 ? v : best + v;
             }
-            best = wave_max(best);
 #pragma unroll
             for (int i = 0; i < kSlots; ++i)
                 if (lane + i * kWave == g) mine[i] = best;
@@ -166,13 +189,14 @@ __device__ inline void route_row(int row, int lane, const float* __restrict__ lo
             weight[static_cast<long>(row) * places + n] = got;
         }
     }
-    const float denom = picked_sum + 1e-20f;
+    const float denom = rule.renorm ? picked_sum + 1e-20f : 1.0f;
     if (lane < top && lane < kWave) {
         chosen[static_cast<long>(row) * places + lane] = my_e >= shift_from ? my_e + always : my_e;
-        weight[static_cast<long>(row) * places + lane] = my_s / denom;
+        weight[static_cast<long>(row) * places + lane] = my_s / denom * rule.scale;
     }
     if (top > kWave && lane == 0)
-        for (int n = kWave; n < top; ++n) weight[static_cast<long>(row) * places + n] /= denom;
+        for (int n = kWave; n < top; ++n)
+            weight[static_cast<long>(row) * places + n] = weight[static_cast<long>(row) * places + n] / denom * rule.scale;
     for (int i = lane; i < always; i += kWave) {
         chosen[static_cast<long>(row) * places + top + i] = shift_from + i;
         weight[static_cast<long>(row) * places + top + i] = 1.0f;
@@ -181,10 +205,10 @@ __device__ inline void route_row(int row, int lane, const float* __restrict__ lo
 
 __global__ void __launch_bounds__(kWave)
 route_topk_kernel(const float* __restrict__ logits, AnyVec correction, int* __restrict__ chosen, float* __restrict__ weight,
-                  int total, int top, int group_count, int group_keep) {
-    if (total <= kWave) route_row<1>(blockIdx.x, threadIdx.x, logits, correction, chosen, weight, total, top, group_count, group_keep);
-    else if (total <= 2 * kWave) route_row<2>(blockIdx.x, threadIdx.x, logits, correction, chosen, weight, total, top, group_count, group_keep);
-    else route_row<kRouteSlots>(blockIdx.x, threadIdx.x, logits, correction, chosen, weight, total, top, group_count, group_keep);
+                  int total, int top, int group_count, int group_keep, RouteRule rule) {
+    if (total <= kWave) route_row<1>(blockIdx.x, threadIdx.x, logits, correction, chosen, weight, total, top, group_count, group_keep, rule);
+    else if (total <= 2 * kWave) route_row<2>(blockIdx.x, threadIdx.x, logits, correction, chosen, weight, total, top, group_count, group_keep, rule);
+    else route_row<kRouteSlots>(blockIdx.x, threadIdx.x, logits, correction, chosen, weight, total, top, group_count, group_keep, rule);
 }
 
 // One workgroup.  counts and places live in shared memory (experts <= 1024).
@@ -233,15 +257,15 @@ moe_plan_kernel(const int* __restrict__ chosen, int pairs, int experts, int* __r
 __global__ void __launch_bounds__(1024)
 route_plan_kernel(const float* __restrict__ logits, AnyVec correction, int* __restrict__ chosen, float* __restrict__ weight,
                   int rows, int total, int top, int group_count, int group_keep, int experts, int* __restrict__ tile_expert,
-                  int* __restrict__ tile_pairs, int max_tiles, int tile, int always) {
+                  int* __restrict__ tile_pairs, int max_tiles, int tile, int always, RouteRule rule) {
     const int routed = experts - always;               // experts the router chooses among; the others every row takes
     __shared__ int count[1024];
     __shared__ int first_tile[1024];
     for (int row = threadIdx.x / kWave; row < rows; row += 1024 / kWave) {
         const int lane = threadIdx.x % kWave;
-        if (total <= kWave) route_row<1>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep, routed, always);
-        else if (total <= 2 * kWave) route_row<2>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep, routed, always);
-        else route_row<kRouteSlots>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep, routed, always);
+        if (total <= kWave) route_row<1>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep, rule, routed, always);
+        else if (total <= 2 * kWave) route_row<2>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep, rule, routed, always);
+        else route_row<kRouteSlots>(row, lane, logits, correction, chosen, weight, total, top, group_count, group_keep, rule, routed, always);
     }
     __syncthreads();                                   // the choices are written; the same workgroup reads them
     plan_tiles(chosen, rows * (top + always), experts, tile_expert, tile_pairs, max_tiles, tile, count, first_tile);
@@ -288,7 +312,7 @@ template <typename T, bool kGated>
 __global__ void __launch_bounds__(kMoeThreads)
 moe_product_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __restrict__ y, const float* __restrict__ pair_weight,
                    const int* __restrict__ tile_expert, const int* __restrict__ tile_pairs, int top, int n, int k, int act,
-                   int runs) {
+                   float limit, int runs) {
     const int tile = blockIdx.x;
     const int e = tile_expert[tile];
     if (e < 0) return;
@@ -359,7 +383,7 @@ moe_product_kernel(const T* __restrict__ x, const T* __restrict__ w, void* __res
             if (q == p) which = pair[q];
         if (col < n && which >= 0) {
             if constexpr (kGated)
-                static_cast<T*>(y)[static_cast<long>(which) * n + col] = from_float<T>(gate_act(mine, act) * mine2);
+                static_cast<T*>(y)[static_cast<long>(which) * n + col] = from_float<T>(glu_value(mine, mine2, act, limit));
             else
                 static_cast<float*>(y)[static_cast<long>(which) * n + col] = mine * pair_weight[which];
         }
@@ -387,7 +411,7 @@ template <int kPB, int kRT, bool kGated>
 __global__ void __launch_bounds__(kMoeThreads)
 moe_product_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y,
                         const float* __restrict__ pair_weight, const int* __restrict__ tile_expert,
-                        const int* __restrict__ tile_pairs, int top, int n, int k, int act) {
+                        const int* __restrict__ tile_pairs, int top, int n, int k, int act, float limit) {
     // kPB blocks of 16 pairs a tile; kRT blocks of 16 rows a wave (a workgroup takes 64 * kRT rows): the more of
     // both, the fewer times the rows of the matrix and of x are fetched again by other workgroups.
     constexpr int kTile = 16 * kPB;
@@ -468,7 +492,7 @@ moe_product_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__
                 if (r >= n) continue;
                 if constexpr (kGated)
                     static_cast<bf16_t*>(y)[static_cast<long>(pair[b]) * n + r] =
-                        from_float<bf16_t>(gate_act(acc[t][b][j], act) * acc2[t][b][j]);
+                        from_float<bf16_t>(glu_value(acc[t][b][j], acc2[t][b][j], act, limit));
                 else
                     static_cast<float*>(y)[static_cast<long>(pair[b]) * n + r] = acc[t][b][j] * scale;
             }
@@ -491,7 +515,7 @@ template <bool kGated>
 __global__ void __launch_bounds__(kMoeThreads, 2)
 moe_product_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ y,
                          const float* __restrict__ pair_weight, const int* __restrict__ tile_expert,
-                         const int* __restrict__ tile_pairs, int top, int n, int k, int act, int n_tiles, int n_blocks) {
+                         const int* __restrict__ tile_pairs, int top, int n, int k, int act, float limit, int n_tiles, int n_blocks) {
     constexpr int kWRows = kGated ? 2 * kBigRows : kBigRows;          // rows of the matrix in a chunk
     constexpr int kXPieces = kBigPairs * 8 / kMoeThreads;             // 16-byte pieces of x a thread brings per chunk
     constexpr int kWPieces = kWRows * 8 / kMoeThreads;
@@ -596,10 +620,10 @@ moe_product_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict_
             if (r >= n) continue;
             float v0, v1, v2, v3;
             if constexpr (kGated) {
-                v0 = gate_act(acc[ta][tb][0], act) * acc2[ta][tb][0];
-                v1 = gate_act(acc[ta][tb][1], act) * acc2[ta][tb][1];
-                v2 = gate_act(acc[ta][tb][2], act) * acc2[ta][tb][2];
-                v3 = gate_act(acc[ta][tb][3], act) * acc2[ta][tb][3];
+                v0 = glu_value(acc[ta][tb][0], acc2[ta][tb][0], act, limit);
+                v1 = glu_value(acc[ta][tb][1], acc2[ta][tb][1], act, limit);
+                v2 = glu_value(acc[ta][tb][2], acc2[ta][tb][2], act, limit);
+                v3 = glu_value(acc[ta][tb][3], acc2[ta][tb][3], act, limit);
                 bf16_t* to = static_cast<bf16_t*>(y) + static_cast<long>(pair) * n + r;
                 if (r + 3 < n && n % 4 == 0) {
                     uint2 packed;
@@ -663,8 +687,11 @@ extern "C" int leone_moe_tile_pairs() { return kTilePairs; }
 extern "C" int leone_route_max_outputs() { return kRouteSlots * kWave; }
 
 extern "C" int leone_route_topk(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight,
-                                int rows, int total, int top, int group_count, int group_keep, hipStream_t stream) {
+                                int rows, int total, int top, int group_count, int group_keep, int score, int group_best,
+                                int renorm, float weight_scale, hipStream_t stream) {
     LEONE_REQUIRE(logits && chosen && weight, "route_topk: null pointer");
+    LEONE_REQUIRE((score == 0 || score == 1) && group_best >= 1 && (renorm == 0 || renorm == 1),
+                  "route_topk: score kind %d, %d best of a group, renorm %d", score, group_best, renorm);
     LEONE_REQUIRE(rows > 0 && total > 0 && total <= kRouteSlots * kWave, "route_topk: rows %d, %d router outputs (at most %d)",
                   rows, total, kRouteSlots * kWave);
     LEONE_REQUIRE(top > 0 && top <= total, "route_topk: %d of %d outputs", top, total);
@@ -672,7 +699,7 @@ extern "C" int leone_route_topk(const float* logits, const void* correction, int
     LEONE_REQUIRE(group_count >= 1 && total % group_count == 0 && group_keep >= 1 && group_keep <= group_count,
                   "route_topk: %d groups (dividing %d outputs), %d kept", group_count, total, group_keep);
     route_topk_kernel<<<rows, kWave, 0, stream>>>(logits, AnyVec{correction, correction_dtype}, chosen, weight, total, top,
-                                                  group_count, group_keep);
+                                                  group_count, group_keep, RouteRule{score, group_best, renorm, weight_scale});
     LEONE_LAUNCH_CHECK("route_topk");
     return 0;
 }
@@ -683,7 +710,10 @@ extern "C" int leone_route_topk(const float* logits, const void* correction, int
 // experts - always on in the router's numbering) is numbered from `experts` on.
 extern "C" int leone_route_plan(const float* logits, const void* correction, int correction_dtype, int* chosen, float* weight,
                                 int rows, int total, int top, int group_count, int group_keep, int experts, int* tile_expert,
-                                int* tile_pairs, int max_tiles, int tile, int always, hipStream_t stream) {
+                                int* tile_pairs, int max_tiles, int tile, int always, int score, int group_best, int renorm,
+                                float weight_scale, hipStream_t stream) {
+    LEONE_REQUIRE((score == 0 || score == 1) && group_best >= 1 && (renorm == 0 || renorm == 1),
+                  "route_plan: score kind %d, %d best of a group, renorm %d", score, group_best, renorm);
     LEONE_REQUIRE(always >= 0 && always < experts, "route_plan: %d of %d experts for every row", always, experts);
     LEONE_REQUIRE(logits && chosen && weight && tile_expert && tile_pairs, "route_plan: null pointer");
     LEONE_REQUIRE(rows > 0 && rows <= 256 && total > 0 && total <= kRouteSlots * kWave, "route_plan: rows %d (at most 256), %d router outputs",
@@ -699,7 +729,8 @@ extern "C" int leone_route_plan(const float* logits, const void* correction, int
     LEONE_REQUIRE(max_tiles >= (needed < pairs ? needed : pairs), "route_plan: %d tiles cannot hold %ld pairs of %d experts", max_tiles,
                   pairs, experts);
     route_plan_kernel<<<1, 1024, 0, stream>>>(logits, AnyVec{correction, correction_dtype}, chosen, weight, rows, total, top,
-                                              group_count, group_keep, experts, tile_expert, tile_pairs, max_tiles, tile, always);
+                                              group_count, group_keep, experts, tile_expert, tile_pairs, max_tiles, tile, always,
+                                              RouteRule{score, group_best, renorm, weight_scale});
     LEONE_LAUNCH_CHECK("route_plan");
     return 0;
 }
@@ -723,19 +754,19 @@ extern "C" int leone_moe_plan(const int* chosen, int pairs, int experts, int* ti
 // size; 16 or 64 for the matrix-core kernel (bfloat16, n and k multiples of 8).
 extern "C" int leone_moe_product(const void* x, const void* w, void* y, const float* pair_weight, int dtype, int gated,
                                  const int* tile_expert, const int* tile_pairs, int max_tiles, int tile, int top, int n, int k,
-                                 int act, hipStream_t stream) {
+                                 int act, float limit, hipStream_t stream) {
     if (tile != kTilePairs) {
         LEONE_REQUIRE(tile == 16 || tile == 64 || tile == 128, "moe_product: tiles of %d pairs", tile);
         LEONE_REQUIRE(dtype == kBF16 && k % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0,
                       "moe_product: the matrix-core kernel takes bfloat16 with an inner size that is a multiple of 8, not %d", k);
         LEONE_REQUIRE(x && w && y && tile_expert && tile_pairs && (gated || pair_weight), "moe_product: null pointer");
         LEONE_REQUIRE(max_tiles > 0 && top > 0 && n > 0 && k > 0, "moe_product: %d tiles, sizes %d x %d", max_tiles, n, k);
-        LEONE_REQUIRE(act == kGateSilu || act == kGateGeluTanh, "moe_product: unknown activation %d", act);
+        LEONE_REQUIRE(act == kGateSilu || act == kGateGeluTanh || (act == kGateClampedSwish && limit > 0.f), "moe_product: unknown activation %d (limit %g)", act, limit);
         const dim3 cores(max_tiles, ceil_div(n, tile == 128 ? 128 : 64));
         LEONE_REQUIRE(cores.y <= 65535, "moe_product: %d rows of a matrix are too many", n);
 #define LEONE_MOE_CORES(PB, RT, G)                                                                                      \
     moe_product_mfma_kernel<PB, RT, G><<<cores, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), \
-                                                                          y, pair_weight, tile_expert, tile_pairs, top, n, k, act)
+                                                                          y, pair_weight, tile_expert, tile_pairs, top, n, k, act, limit)
         if (tile == 16) {
             if (gated) LEONE_MOE_CORES(1, 1, true);
             else LEONE_MOE_CORES(1, 1, false);
@@ -748,11 +779,11 @@ extern "C" int leone_moe_product(const void* x, const void* w, void* y, const fl
             const int grid = static_cast<int>((places + 7) / 8 * 8);
             if (gated)
                 moe_product_tiled_kernel<true><<<grid, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w),
-                                                                                 y, pair_weight, tile_expert, tile_pairs, top, n, k, act,
+                                                                                 y, pair_weight, tile_expert, tile_pairs, top, n, k, act, limit,
                                                                                  static_cast<int>(cores.x), static_cast<int>(cores.y));
             else
                 moe_product_tiled_kernel<false><<<grid, kMoeThreads, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w),
-                                                                                  y, pair_weight, tile_expert, tile_pairs, top, n, k, act,
+                                                                                  y, pair_weight, tile_expert, tile_pairs, top, n, k, act, limit,
                                                                                   static_cast<int>(cores.x), static_cast<int>(cores.y));
         }
 #undef LEONE_MOE_CORES
@@ -762,14 +793,14 @@ extern "C" int leone_moe_product(const void* x, const void* w, void* y, const fl
     LEONE_REQUIRE(dtype == kF32 || dtype == kBF16, "moe_product: unknown element type %d", dtype);
     LEONE_REQUIRE(x && w && y && tile_expert && tile_pairs && (gated || pair_weight), "moe_product: null pointer");
     LEONE_REQUIRE(max_tiles > 0 && top > 0 && n > 0 && k > 0, "moe_product: %d tiles, sizes %d x %d", max_tiles, n, k);
-    LEONE_REQUIRE(act == kGateSilu || act == kGateGeluTanh, "moe_product: unknown activation %d", act);
+    LEONE_REQUIRE(act == kGateSilu || act == kGateGeluTanh || (act == kGateClampedSwish && limit > 0.f), "moe_product: unknown activation %d (limit %g)", act, limit);
     const uintptr_t run = 8 * (dtype == kF32 ? sizeof(float) : sizeof(bf16_t));
     const int runs = k % 8 == 0 && reinterpret_cast<uintptr_t>(x) % run == 0 && reinterpret_cast<uintptr_t>(w) % run == 0;
     const dim3 grid(max_tiles, ceil_div(n, kMoeCols));
     LEONE_REQUIRE(grid.y <= 65535, "moe_product: %d rows of a matrix are too many", n);
 #define LEONE_MOE(T, G)                                                                                                   \
     moe_product_kernel<T, G><<<grid, kMoeThreads, 0, stream>>>(static_cast<const T*>(x), static_cast<const T*>(w), y, pair_weight, \
-                                                               tile_expert, tile_pairs, top, n, k, act, runs)
+                                                               tile_expert, tile_pairs, top, n, k, act, limit, runs)
     if (dtype == kF32) {
         if (gated) LEONE_MOE(float, true);
         else LEONE_MOE(float, false);

@@ -1462,12 +1462,48 @@ def add_normed(x: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional[to
     return x if same else y
 
 
+ROUTER_SCORES = {"softmax": 0, "sigmoid": 1}     # how a router turns its logits into scores
+# what experts put on gate and up: a gate activation, or "clamped_swish" (gate and up held to a limit, see ``glu_value``)
+EXPERT_ACTIVATIONS = {**GATE_ACTIVATIONS, "clamped_swish": 2}
+
+
+class RouterRule:
+    """How a router scores and weighs (the defaults are a softmax router whose winners' scores are renormalised):
+    ``score`` "softmax" over all outputs or "sigmoid" of each; ``group_best``: a group's score is the sum of its so
+    many best choice scores; ``renormalize``: the winners' scores over their sum, else the scores themselves;
+    ``scale`` multiplies the weights."""
+
+    def __init__(self, score: str = "softmax", group_best: int = 1, renormalize: bool = True, scale: float = 1.0):
+        if score not in ROUTER_SCORES:
+            raise KernelError(f"unknown router score {score!r}; known: {', '.join(ROUTER_SCORES)}")
+        if int(group_best) < 1:
+            raise KernelError(f"a group's score is made of at least one of its outputs, not {group_best}")
+        self.score, self.group_best, self.renormalize, self.scale = score, int(group_best), bool(renormalize), float(scale)
+
+    def args(self) -> tuple:
+        return ROUTER_SCORES[self.score], self.group_best, 1 if self.renormalize else 0, self.scale
+
+
+_DEFAULT_RULE = RouterRule()
+
+
+def _expert_act(activation: str, limit: Optional[float]) -> tuple:
+    try:
+        code = EXPERT_ACTIVATIONS[activation]
+    except KeyError:
+        raise KernelError(f"unknown expert activation {activation!r}; known: {', '.join(EXPERT_ACTIVATIONS)}") from None
+    if code == 2 and not (limit is not None and limit > 0.0):
+        raise KernelError(f"the clamped activation needs a positive limit, found {limit!r}")
+    return code, float(limit or 0.0)
+
+
 def route_topk(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, group_count: int = 1,
-               group_keep: int = 1) -> tuple:
-    """The router's choice for every row of float32 ``logits [rows, outputs]``: scores softmax(logits); choice scores
-    with ``correction`` added; the outputs form ``group_count`` equal groups of neighbours of which the
-    ``group_keep`` with the best choice score stay open; the ``top`` best open outputs win.  Returns their
-    indices (int32 ``[rows, top]``, best first) and their scores over the winners' sum (float32)."""
+               group_keep: int = 1, rule: Optional[RouterRule] = None) -> tuple:
+    """The router's choice for every row of float32 ``logits [rows, outputs]``: scores softmax(logits) (or what
+    ``rule`` says); choice scores with ``correction`` added; the outputs form ``group_count`` equal groups of
+    neighbours of which the ``group_keep`` with the best group score stay open; the ``top`` best open outputs win.
+    Returns their indices (int32 ``[rows, top]``, best first) and their weights (float32): by default their scores
+    over the winners' sum."""
     rows, total = logits.shape
     if total > library().leone_route_max_outputs():
         raise KernelError(f"route_topk: {total} router outputs, the kernel takes {library().leone_route_max_outputs()}")
@@ -1475,7 +1511,8 @@ def route_topk(logits: torch.Tensor, correction: Optional[torch.Tensor], top: in
     weight = torch.empty((rows, top), dtype=torch.float32, device=logits.device)
     call("leone_route_topk", _dev(logits, "router logits", torch.float32),
          _dev(correction, "router correction", None, (total,)), _code(correction, "router correction") if correction is not None else F32,
-         _dev(chosen, "chosen"), _dev(weight, "weights"), rows, total, int(top), int(group_count), int(group_keep), _stream())
+         _dev(chosen, "chosen"), _dev(weight, "weights"), rows, total, int(top), int(group_count), int(group_keep),
+         *(rule or _DEFAULT_RULE).args(), _stream())
     return chosen, weight
 
 
@@ -1506,8 +1543,9 @@ def _check_experts(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tenso
     return rows, hidden, experts, ff
 
 
-def _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra) -> torch.Tensor:
+def _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra, limit=None) -> torch.Tensor:
     rows, hidden, experts, ff = _check_experts(x, w_gate_up, w_down)
+    act, limit = _expert_act(activation, limit)
     top = chosen.shape[1]
     pairs = rows * top
     tile, max_tiles, tile_expert, tile_pairs = tiles
@@ -1515,11 +1553,11 @@ def _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, ex
     hidden_act = torch.empty((pairs, ff), dtype=x.dtype, device=device)
     call("leone_moe_product", _dev(x, "routed rows"), _dev(w_gate_up, "expert gate/up"), _dev(hidden_act, "expert hidden"), 0,
          _code(x, "routed rows"), 1, _dev(tile_expert, "tiles"), _dev(tile_pairs, "tile pairs"), max_tiles, tile, top, ff, hidden,
-         _gate_code(activation), _stream())
+         act, limit, _stream())
     pair_out = torch.empty((pairs, hidden), dtype=torch.float32, device=device)
     call("leone_moe_product", _dev(hidden_act, "expert hidden"), _dev(w_down, "expert down"), _dev(pair_out, "pair results"),
          _dev(weight, "weights", torch.float32, (rows, top)), _code(x, "routed rows"), 0, _dev(tile_expert, "tiles"),
-         _dev(tile_pairs, "tile pairs"), max_tiles, tile, top, hidden, ff, 0, _stream())
+         _dev(tile_pairs, "tile pairs"), max_tiles, tile, top, hidden, ff, 0, 0.0, _stream())
     out = torch.empty((rows, hidden), dtype=torch.float32, device=device)
     call("leone_moe_combine", _dev(pair_out, "pair results"), _dev(chosen, "chosen"), _dev(weight, "weights"),
          _dev(x, "routed rows"), _code(x, "routed rows"), _dev(extra, "extra", torch.float32, (rows, hidden)),
@@ -1528,7 +1566,8 @@ def _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, ex
 
 
 def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, w_gate_up: torch.Tensor,
-                   w_down: torch.Tensor, activation: str = "silu", extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   w_down: torch.Tensor, activation: str = "silu", extra: Optional[torch.Tensor] = None,
+                   limit: Optional[float] = None) -> torch.Tensor:
     """Every row through the experts chosen for it: float32 ``[rows, hidden]`` = sum over a row's places of
     weight * W_down[e] (act(W_gate[e] x) * (W_up[e] x)), in the places' order; a chosen index from the number of
     experts on stands for an expert that hands the row on as it is; ``extra`` (float32 ``[rows, hidden]``) is added.
@@ -1539,12 +1578,13 @@ def routed_experts(x: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor, 
     tiles = _expert_tiles(x, rows, top, experts, hidden, ff)
     call("leone_moe_plan", _dev(chosen, "chosen", torch.int32, (rows, top)), rows * top, experts, _dev(tiles[2], "tiles"),
          _dev(tiles[3], "tile pairs"), tiles[1], tiles[0], _stream())
-    return _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra)
+    return _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra, limit)
 
 
 def routed_feed_forward(x: torch.Tensor, logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, group_count: int,
                         group_keep: int, w_gate_up: torch.Tensor, w_down: torch.Tensor, activation: str = "silu",
-                        extra: Optional[torch.Tensor] = None, always: int = 0) -> torch.Tensor:
+                        extra: Optional[torch.Tensor] = None, always: int = 0, rule: Optional[RouterRule] = None,
+                        limit: Optional[float] = None) -> torch.Tensor:
     """``route_topk`` on the router's float32 ``logits`` and ``routed_experts`` with its choice; for steps of few rows
     (up to ``ROUTE_PLAN_ROWS``) the choice and the tiles are made in one launch.  ``always`` (such steps only): the
     last so many experts of the matrices are no choice of the router's but taken by every row with weight 1 (a
@@ -1554,8 +1594,8 @@ def routed_feed_forward(x: torch.Tensor, logits: torch.Tensor, correction: Optio
     if rows > ROUTE_PLAN_ROWS:
         if always:
             raise KernelError(f"routed_feed_forward: experts for every row ride along in steps of up to {ROUTE_PLAN_ROWS} rows only")
-        chosen, weight = route_topk(logits, correction, top, group_count, group_keep)
-        return routed_experts(x, chosen, weight, w_gate_up, w_down, activation, extra)
+        chosen, weight = route_topk(logits, correction, top, group_count, group_keep, rule)
+        return routed_experts(x, chosen, weight, w_gate_up, w_down, activation, extra, limit)
     if total > library().leone_route_max_outputs():
         raise KernelError(f"route_topk: {total} router outputs, the kernel takes {library().leone_route_max_outputs()}")
     if not 0 <= always < experts:
@@ -1567,5 +1607,198 @@ def routed_feed_forward(x: torch.Tensor, logits: torch.Tensor, correction: Optio
     call("leone_route_plan", _dev(logits, "router logits", torch.float32, (rows, total)),
          _dev(correction, "router correction", None, (total,)), _code(correction, "router correction") if correction is not None else F32,
          _dev(chosen, "chosen"), _dev(weight, "weights"), rows, total, int(top), int(group_count), int(group_keep), experts,
-         _dev(tiles[2], "tiles"), _dev(tiles[3], "tile pairs"), tiles[1], tiles[0], int(always), _stream())
-    return _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra)
+         _dev(tiles[2], "tiles"), _dev(tiles[3], "tile pairs"), tiles[1], tiles[0], int(always),
+         *(rule or _DEFAULT_RULE).args(), _stream())
+    return _expert_products(x, chosen, weight, tiles, w_gate_up, w_down, activation, extra, limit)
+
+
+# ---- a forget gate per key channel, attention through a shared latent, the stream as a sum over depth -----------
+GATED_CHUNKS = (64, 256)     # rows of a chunk and the portions that are walked in chunks (as ``OUTER_CHUNKS``)
+
+
+def gated_scan(proj: torch.Tensor, columns: dict, f_bias: torch.Tensor, lower: torch.Tensor, state: torch.Tensor, step,
+               heads: int, dim: int, vdim: int, q_activation: Optional[str] = "silu", write_state: bool = True) -> torch.Tensor:
+    """The matrix memory whose forget gate also says what is written, over every entry's rows: per head and key
+    channel f = lower + (1 - lower) sigmoid(pre + f_bias); S <- diag(f) S + (1 - f) v^T; o = S^T q with q = act(q_pre).
+    ``proj`` float32 ``[rows, width]`` holds q_pre, the gates' pre (``heads * dim`` each) and v (``heads * vdim``) at
+    ``columns`` "q", "f", "v"; ``f_bias`` and ``lower`` ``[heads * dim]`` of one type; ``state`` float32
+    ``[slots, heads, dim * vdim]``.  Returns o float32 ``[rows, heads * vdim]``.  Long portions are walked in chunks
+    side by side, as in ``outer_scan``, the chunks chained by the product of their gates per key channel."""
+    rows, width = proj.shape
+    if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (heads, dim * vdim) or not state.is_contiguous():
+        raise KernelError(f"gated_scan: state {tuple(state.shape)} is not [slots, {heads}, {dim * vdim}] float32")
+    if f_bias.dtype != lower.dtype:
+        raise KernelError("gated_scan: the gates' bias and lower bound must share one type")
+    if q_activation not in (None, "silu"):
+        raise KernelError(f"gated_scan: queries pass as they are or through silu, not {q_activation!r}")
+    spans = entry_spans(step)
+    device = proj.device
+    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=device)
+
+    def walk(segments, state_in, state_out, no_input=False, accumulate=False, product=None):
+        call("leone_gated_scan", _dev(proj, "projection", torch.float32), width, columns["q"], columns["f"], columns["v"],
+             _dev(f_bias, "gate bias", None, (heads * dim,)), _dev(lower, "lower bound", None, (heads * dim,)),
+             _code(f_bias, "gate bias"), 1 if q_activation == "silu" else 0, 1 if no_input else 0, 1 if accumulate else 0,
+             _dev(segments, "segments", torch.int32), segments.shape[0],
+             _dev(state_in, "state read"), state_in.stride(0) if state_in is not None else 0,
+             _dev(state_out, "state written"), state_out.stride(0) if state_out is not None else 0,
+             _dev(product, "gate products"), _dev(out, "out"), heads, dim, vdim, _stream())
+
+    plan = chunk_plan(step, *GATED_CHUNKS)
+    if plan is None:
+        walk(spans, state, state if write_state else None)
+    else:
+        chunks = plan["chunks"]
+        work = torch.empty((chunks.shape[0], heads, dim * vdim), dtype=torch.float32, device=device)
+        product = torch.empty((chunks.shape[0], heads, dim), dtype=torch.float32, device=device)
+        walk(chunks, None, work, product=product)
+        call("leone_gated_chain", _dev(plan["links"], "links", torch.int32), plan["links"].shape[0], _dev(work, "work"),
+             work.stride(0), _dev(product, "gate products"), _dev(state, "state"), state.stride(0), heads, dim, vdim,
+             1 if write_state else 0, _stream())
+        walk(plan["again"], work, None, no_input=True, accumulate=True)
+        if plan["short"].shape[0]:
+            walk(plan["short"], state, state if write_state else None)
+    return out
+
+
+def _rotation_tables(what: str, part: int, cos, sin):
+    """(address of cos, of sin, pairs, table positions) of a rotation of neighbouring pairs on the first elements of a
+    part of ``part`` elements."""
+    if cos is None:
+        return 0, 0, 0, 1
+    if sin is None or sin.shape != cos.shape or cos.dim() != 2 or 2 * cos.shape[1] > part:
+        raise KernelError(f"{what}: cos and sin tables must both be [positions, pairs] with 2 * pairs <= {part}")
+    return _dev(cos, "rope cos", torch.float32), _dev(sin, "rope sin", torch.float32), cos.shape[1], cos.shape[0]
+
+
+def latent_prepare(proj: torch.Tensor, out_dtype: torch.dtype, eps: float, *, q_column: Optional[int] = None, q_rank: int = 0,
+                   q_gain: Optional[torch.Tensor] = None, kv_column: Optional[int] = None, rank: int = 0, rot: int = 0,
+                   kv_gain: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
+                   sin: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
+                   row_entry: Optional[torch.Tensor] = None, block_table: Optional[torch.Tensor] = None,
+                   pool: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """From the float32 down-projections ``proj [rows, width]``: the query latent (``q_rank`` columns from
+    ``q_column``) RMS-normed times ``q_gain`` comes back in ``out_dtype``; the key/value latent (``rank`` columns from
+    ``kv_column``) RMS-normed times ``kv_gain`` and the ``rot`` columns behind it, rotated in neighbouring pairs by the
+    row's position, are written into ``pool [pages, page_tokens, rank + rot]`` at the row's place.  Either half may be
+    left out."""
+    rows, width = proj.shape
+    q_out = torch.empty((rows, q_rank), dtype=out_dtype, device=proj.device) if q_column is not None else None
+    gains = [g for g in (q_gain, kv_gain) if g is not None]
+    if not gains or len({g.dtype for g in gains}) != 1:
+        raise KernelError("latent_prepare: the gains must come in one type")
+    page_tokens = max_blocks = 0
+    if kv_column is not None:
+        if pool is None or pool.dim() != 3 or pool.shape[2] != rank + rot or pool.dtype != out_dtype:
+            raise KernelError(f"latent_prepare: the pool must be {out_dtype} [pages, page_tokens, {rank + rot}], found "
+                              f"{None if pool is None else (pool.dtype, tuple(pool.shape))}")
+        if block_table is None or positions is None or row_entry is None:
+            raise KernelError("latent_prepare: a cache write needs positions, a row map and a block table")
+        page_tokens, max_blocks = pool.shape[1], block_table.shape[1]
+    cos_at, sin_at, pairs, table_positions = _rotation_tables("latent_prepare", rot, cos, sin)
+    call("leone_latent_prepare", _dev(proj, "projection", torch.float32), width, rows,
+         -1 if q_column is None else int(q_column), int(q_rank), _dev(q_gain, "query gain", None, (q_rank,)) if q_column is not None else 0,
+         _dev(q_out, "query latent"), -1 if kv_column is None else int(kv_column), int(rank), int(rot),
+         _dev(kv_gain, "latent gain", None, (rank,)) if kv_column is not None else 0, _code(gains[0], "gain"), float(eps),
+         cos_at, sin_at, pairs, table_positions,
+         _dev(positions, "positions", torch.int32, (rows,)) if kv_column is not None else 0,
+         _dev(row_entry, "row map", torch.int32, (rows,)) if kv_column is not None else 0,
+         _dev(block_table, "block table", torch.int32) if kv_column is not None else 0, max_blocks, page_tokens,
+         _dev(pool, "latent pool") if kv_column is not None else 0, _CODES[out_dtype], _stream())
+    return q_out
+
+
+def head_product(x: torch.Tensor, weight: torch.Tensor, heads: int, out_dtype: torch.dtype, *, tail: int = 0,
+                 cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                 positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """A product a head: ``x`` float32 ``[rows, heads * (inner + tail)]``, ``weight`` ``[heads, inner, outer]`` ->
+    ``[rows, heads * (outer + tail)]`` in ``out_dtype`` with y[r, h, :outer] = x[r, h, :inner] weight[h].  The ``tail``
+    elements behind a head's inner ones are handed on behind its outer ones, rotated in neighbouring pairs by the
+    row's position if tables come."""
+    rows = x.shape[0]
+    if weight.dim() != 3 or weight.shape[0] != heads or x.dim() != 2 or x.shape[1] != heads * (weight.shape[1] + tail):
+        raise KernelError(f"head_product: rows {tuple(x.shape)} against {tuple(weight.shape)} for {heads} heads with a tail of {tail}")
+    inner, outer = weight.shape[1], weight.shape[2]
+    out = torch.empty((rows, heads * (outer + tail)), dtype=out_dtype, device=x.device)
+    cos_at, sin_at, pairs, table_positions = _rotation_tables("head_product", tail, cos, sin)
+    call("leone_head_product", _dev(x, "head rows", torch.float32), x.shape[1], inner + tail, _dev(weight, "head matrices"),
+         _code(weight, "head matrices"), _dev(out, "head results"), _CODES[out_dtype], out.shape[1], outer + tail, rows, heads,
+         inner, outer, int(tail), cos_at, sin_at, pairs, table_positions,
+         _dev(positions, "positions", torch.int32, (rows,)) if cos is not None else 0, _stream())
+    return out
+
+
+def latent_attention(q: torch.Tensor, pool: torch.Tensor, positions: torch.Tensor, row_entry: torch.Tensor,
+                     block_table: torch.Tensor, heads: int, rank: int, rot: int, scale: float, window: int = 0) -> torch.Tensor:
+    """Softmax attention over a cache of latents shared by the heads: ``q`` float32 ``[rows, heads * (rank + rot)]`` (the
+    keys' up-projection already on the query's side, see ``head_product``), ``pool`` ``[pages, page_tokens, rank + rot]``;
+    a row sees the latents of its request at positions pos - window < j <= pos (``window`` 0: all).  Returns float32
+    ``[rows, heads * rank]``: every head's weighted sum of the latents' first ``rank`` elements."""
+    rows = q.shape[0]
+    if pool.dim() != 3 or pool.shape[2] != rank + rot or q.shape[1] != heads * (rank + rot):
+        raise KernelError(f"latent_attention: queries {tuple(q.shape)} and pool {tuple(pool.shape)} do not fit {heads} heads of {rank} + {rot}")
+    if rank + rot > library().leone_latent_max_width():
+        raise KernelError(f"latent_attention: a latent of {rank} + {rot} elements, the kernel takes {library().leone_latent_max_width()}")
+    out = torch.empty((rows, heads * rank), dtype=torch.float32, device=q.device)
+    call("leone_latent_attention", _dev(q, "latent queries", torch.float32), _dev(out, "latent sums"), _dev(pool, "latent pool"),
+         _code(pool, "latent pool"), _dev(positions, "positions", torch.int32, (rows,)),
+         _dev(row_entry, "row map", torch.int32, (rows,)), _dev(block_table, "block table", torch.int32), block_table.shape[1],
+         rows, heads, int(rank), int(rot), pool.shape[1], float(scale), int(window), _stream())
+    return out
+
+
+class ScaledDelta:
+    """What a sublayer adds to the stream, still to be multiplied by a factor: ``scale * rows`` is meant (``rows``
+    float32 ``[n, hidden]`` or planes ``[p, n, hidden]``).  The norm that runs next takes it in place of a delta
+    (``residual_norm``); any other consumer asks for ``materialize()``."""
+
+    def __init__(self, rows: torch.Tensor, scale: float):
+        self.rows, self.scale = rows, float(scale)
+
+    def materialize(self) -> torch.Tensor:
+        rows = self.rows.sum(dim=0) if self.rows.dim() == 3 else self.rows
+        return rows.float() * self.scale
+
+
+def _planes(delta: Optional[torch.Tensor], n: int, hidden: int, what: str):
+    if delta is None:
+        return None, 1, 0
+    if delta.dtype != torch.float32:
+        delta = delta.float()
+    stacked = delta.dim() == 3
+    planes = delta.shape[0] if stacked else 1
+    _dev(delta, what, torch.float32, (planes, n, hidden) if stacked else (n, hidden))
+    return delta, planes, n * hidden
+
+
+def residual_norm(x: torch.Tensor, delta: Optional[torch.Tensor], scale: float, gain: Optional[torch.Tensor], eps: float,
+                  out_dtype: Optional[torch.dtype], rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x += scale * delta in the float32 stream (``delta`` float32 ``[n, hidden]`` or planes; None: nothing is added), then
+    rmsnorm(x) * gain in ``out_dtype`` (None: no norm, only the sum).  With ``rows`` (int32 indices) only those rows come
+    back and the stream is left as it was."""
+    n, hidden = x.shape
+    delta, planes, plane = _planes(delta, n, hidden, "delta")
+    n_out = n if rows is None else rows.numel()
+    y = torch.empty((n_out, hidden), dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    if delta is None and y is None:
+        return None
+    call("leone_residual_norm", _dev(x, "stream", torch.float32), _dev(delta, "delta"), planes, plane, float(scale),
+         _dev(gain, "gain", None, (hidden,)) if y is not None else 0, _code(gain, "gain") if y is not None else F32, float(eps),
+         _dev(y, "normed rows"), _CODES[out_dtype] if out_dtype is not None else F32,
+         _dev(rows, "rows", torch.int32) if rows is not None else 0, n_out, hidden, _stream())
+    return y
+
+
+def depth_mix(x: torch.Tensor, delta: Optional[torch.Tensor], scale: float, history: torch.Tensor, count: int,
+              weight: torch.Tensor) -> None:
+    """A layer's own result X = x + scale * delta is kept as ``history[count - 1]`` and the stream becomes
+    sum_{j < count} weight[j] * history[j], in place in ``x``.  ``history`` float32 ``[slots, n, hidden]``."""
+    n, hidden = x.shape
+    delta, planes, plane = _planes(delta, n, hidden, "delta")
+    if history.dtype != torch.float32 or history.dim() != 3 or tuple(history.shape[1:]) != (n, hidden) or not 1 <= count <= history.shape[0]:
+        raise KernelError(f"depth_mix: a history {tuple(history.shape)} for {count} results of {tuple(x.shape)}")
+    if weight.numel() != count:
+        raise KernelError(f"depth_mix: {weight.numel()} weights for {count} results")
+    call("leone_depth_mix", _dev(x, "stream", torch.float32), _dev(delta, "delta"), planes, plane, float(scale),
+         _dev(history, "history"), history.stride(0), int(count), _dev(weight, "depth weights"), _code(weight, "depth weights"),
+         n * hidden, _stream())

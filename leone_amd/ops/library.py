@@ -77,11 +77,22 @@ _PROTOTYPES = {
                                     c_int, c_int, P],
     "leone_attention_prefill_kept": [P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P, P,
                                      c_int, c_int, P],
-    "leone_route_topk": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, P],
-    "leone_route_plan": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, c_int, c_int, c_int, P],
+    "leone_route_topk": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, P],
+    "leone_route_plan": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int,
+                         c_float, P],
     "leone_moe_plan": [P, c_int, c_int, P, P, c_int, c_int, P],
-    "leone_moe_product": [P, P, P, P, c_int, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "leone_moe_product": [P, P, P, P, c_int, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, P],
     "leone_moe_combine": [P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, P],
+    "leone_gated_scan": [P, ctypes.c_long, c_int, c_int, c_int, P, P, c_int, c_int, c_int, c_int, P, c_int, P, ctypes.c_long, P,
+                         ctypes.c_long, P, P, c_int, c_int, c_int, P],
+    "leone_gated_chain": [P, c_int, P, ctypes.c_long, P, P, ctypes.c_long, c_int, c_int, c_int, c_int, P],
+    "leone_latent_prepare": [P, ctypes.c_long, c_int, c_int, c_int, P, P, c_int, c_int, c_int, P, c_int, c_float, P, P, c_int, c_int,
+                             P, P, P, c_int, c_int, P, c_int, P],
+    "leone_head_product": [P, ctypes.c_long, ctypes.c_long, P, c_int, P, c_int, ctypes.c_long, ctypes.c_long, c_int, c_int, c_int,
+                           c_int, c_int, P, P, c_int, c_int, P, P],
+    "leone_latent_attention": [P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
+    "leone_residual_norm": [P, P, c_int, ctypes.c_long, c_float, P, c_int, c_float, P, c_int, P, c_int, c_int, P],
+    "leone_depth_mix": [P, P, c_int, ctypes.c_long, c_float, P, ctypes.c_long, c_int, P, c_int, ctypes.c_long, P],
     "leone_delta_chain": [P, c_int, P, ctypes.c_long, P, P, ctypes.c_long, c_int, c_int, c_int, c_int, P],
 }
 
@@ -122,6 +133,8 @@ def library() -> ctypes.CDLL:
             lib.leone_gemm_rows_chunk.argtypes = [c_int]
             lib.leone_moe_tile_pairs.restype = c_int
             lib.leone_moe_tile_pairs.argtypes = []
+            lib.leone_latent_max_width.restype = c_int
+            lib.leone_latent_max_width.argtypes = []
             lib.leone_route_max_outputs.restype = c_int
             lib.leone_route_max_outputs.argtypes = []
             lib.leone_library_product_available.restype = c_int

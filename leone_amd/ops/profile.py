@@ -58,6 +58,13 @@ OPERATIONS = {
     "leone_route_plan": "router",
     "leone_moe_product": "experts",
     "leone_moe_combine": "experts",
+    "leone_gated_scan": "gated scan",
+    "leone_gated_chain": "gated scan",
+    "leone_latent_prepare": "latent norm rope kv",
+    "leone_head_product": "head product",
+    "leone_latent_attention": "attention",
+    "leone_residual_norm": "norm",
+    "leone_depth_mix": "depth mix",
 }
 LIBRARY_PRODUCT = "gemm library"
 ORDER = ["embed", "norm", "gemv fused", "gemm rows", LIBRARY_PRODUCT, "gemm f32", "qknorm rope kv", "attention", "swiglu",

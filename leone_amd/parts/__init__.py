@@ -1,4 +1,4 @@
-from . import block, conv, feedforward, mixer, norm, position, recurrent  # noqa: F401  (register the built-in kinds)
+from . import block, conv, feedforward, latent, mixer, norm, position, recurrent  # noqa: F401  (register the built-in kinds)
 from .base import (BLOCKS, CONVS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, KvNeed, Part, PartSpec, Registry, RowTiling,
                    StateNeed)
 from .context import CacheView, EntryInfo, KvCacheView, StateCacheView, StepContext

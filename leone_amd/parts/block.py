@@ -240,3 +240,66 @@ class PostNormBlock(Part):
             return ops.NormedDelta(mixed, self.norm1)
         h = self.norm1.add_behind(x, mixed, step.dtype)
         return ops.NormedDelta(self.feed_forward.forward(h, step), self.norm2)
+
+
+@BLOCKS.register("scaled_prenorm")
+class ScaledPreNormBlock(Part):
+    """Pre-norm sublayers whose results enter the stream times a factor, the mixer reading through a short convolution:
+
+        x <- x + scale * mixer(conv1(norm1(x)));   x <- x + scale * feed_forward(norm2(x))
+
+    The second sublayer is there only if ``feed_forward`` is given; ``conv1`` may be None (the mixer reads the norm's
+    result as it is).  The convolution keeps its last inputs per request, so the block's cache need is a dict:
+    ``mixer`` (the mixer's own) and ``conv1``.  Parameters: ``norm1``, ``conv1``, ``mixer``, ``scale`` and optionally
+    ``norm2``, ``feed_forward`` (part specs).  The sublayers hand back float32.  The block's last sum is left to
+    whoever runs next (``ops.ScaledDelta``): a norm adds it in its own kernel, and a model that re-mixes the stream
+    over depth takes it into that kernel.
+    """
+
+    def __init__(self, spec: PartSpec, **context):
+        self.norm1 = NORMS.build(spec["norm1"], **context)
+        self.conv1 = CONVS.build(spec["conv1"], **context) if spec.get("conv1") is not None else None
+        self.mixer = MIXERS.build(spec["mixer"], **context)
+        self.feed_forward = FEED_FORWARDS.build(spec["feed_forward"], **context) if spec.get("feed_forward") is not None else None
+        self.norm2 = NORMS.build(spec["norm2"], **context) if spec.get("norm2") is not None else None
+        self.scale = float(spec.get("scale", 1.0))
+        if self.feed_forward is not None and self.norm2 is None:
+            raise ValueError("a scaled_prenorm block with a feed-forward needs norm2")
+
+    def parts(self):
+        return tuple(part for part in (self.norm1, self.conv1, self.mixer, self.norm2, self.feed_forward) if part is not None)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False) for part in self.parts())
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for part in self.parts() for s in part.tensor_specs()]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for part in self.parts():
+            part.bind(tensors)
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [w for part in self.parts() if hasattr(part, "streamed_weights") for w in part.streamed_weights()]
+
+    def cache_need(self):
+        need = {"mixer": self.mixer.cache_need()}
+        if self.conv1 is not None:
+            need["conv1"] = self.conv1.cache_need()
+        return need
+
+    def row_tilings(self):
+        return [part.row_tiling() for part in self.parts() if hasattr(part, "row_tiling")]
+
+    def forward(self, x: torch.Tensor, pending, step: StepContext, cache):
+        cache = cache or {}
+        if self.conv1 is None:
+            h = self.norm1.add_norm(x, pending, step.dtype)
+        else:
+            h = self.conv1.forward(self.norm1.add_norm(x, pending, torch.float32), step, cache.get("conv1"), step.dtype)
+        delta = ops.ScaledDelta(self.mixer.forward(h, step, cache.get("mixer")), self.scale)
+        if self.feed_forward is None:
+            return delta
+        h = self.norm2.add_norm(x, delta, step.dtype)
+        return ops.ScaledDelta(self.feed_forward.forward(h, step), self.scale)

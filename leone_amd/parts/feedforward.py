@@ -110,6 +110,12 @@ class RoutedGluMlp(Part):
     ``correction`` ``[experts + identity]`` (None: no correction) and ``expert`` (a pattern with ``{e}``:
     ``expert.format(e=3) + ".gate"`` and so on), ``shared``.
 
+    Optional, for routers of another rule: ``score`` ("softmax", or "sigmoid": every output's own sigmoid), ``group_best``
+    (a group's score is the sum of its so many best choice scores, 1 by default), ``renormalize`` (False: the weights
+    are the winners' scores themselves), ``weight_scale`` (multiplies the weights), and ``activation`` "clamped_swish"
+    with ``limit`` (``ops.EXPERT_ACTIVATIONS``): g = min(gate, limit), u = clamp(up, -limit, limit),
+    g sigmoid(1.702 g) (u + 1).
+
     The choice lives on the device only: which rows go to which expert is worked out there, and the grids do not
     depend on it, so a recorded step replays with other choices.
     """
@@ -126,8 +132,13 @@ class RoutedGluMlp(Part):
         if self.top > self.total or self.total % self.group_count or not 1 <= self.group_keep <= self.group_count:
             raise ValueError(f"a router of {self.total} outputs cannot choose {self.top} from {self.group_keep} of "
                              f"{self.group_count} equal groups")
-        if self.activation not in ops.GATE_ACTIVATIONS:
-            raise ValueError(f"unknown gate activation {self.activation!r}; known: {', '.join(ops.GATE_ACTIVATIONS)}")
+        if self.activation not in ops.EXPERT_ACTIVATIONS:
+            raise ValueError(f"unknown expert activation {self.activation!r}; known: {', '.join(ops.EXPERT_ACTIVATIONS)}")
+        self.limit = float(p["limit"]) if p.get("limit") is not None else None
+        if self.activation == "clamped_swish" and not (self.limit and self.limit > 0.0):
+            raise ValueError(f"the clamped activation needs a positive limit, found {self.limit!r}")
+        self.rule = ops.RouterRule(str(p.get("score") or "softmax"), int(p.get("group_best") or 1),
+                                   bool(p.get("renormalize", True)), float(p.get("weight_scale", 1.0)))
         self.router_name, self.correction_name, self.expert_name = p["router"], p.get("correction"), p["expert"]
         self.shared = FEED_FORWARDS.build(p["shared"], **context) if p.get("shared") is not None else None
         self.w_router = self.correction = self.w_gate_up = self.w_down = self.w_gate_up_all = self.w_down_all = None
@@ -177,7 +188,8 @@ class RoutedGluMlp(Part):
         logits = ops.linear(y, self.w_router, out_dtype=torch.float32)
         if self.always and y.shape[0] <= ops.ROUTE_PLAN_ROWS:
             return ops.routed_feed_forward(y, logits, self.correction, self.top, self.group_count, self.group_keep,
-                                           self.w_gate_up_all, self.w_down_all, self.activation, always=self.always)
+                                           self.w_gate_up_all, self.w_down_all, self.activation, always=self.always,
+                                           rule=self.rule, limit=self.limit)
         extra = None
         if self.shared is not None:
             extra = self.shared.forward(y, step)
@@ -186,4 +198,5 @@ class RoutedGluMlp(Part):
             if extra.dtype != torch.float32:
                 extra = extra.float()
         return ops.routed_feed_forward(y, logits, self.correction, self.top, self.group_count, self.group_keep,
-                                       self.w_gate_up, self.w_down, self.activation, extra=extra)
+                                       self.w_gate_up, self.w_down, self.activation, extra=extra, rule=self.rule,
+                                       limit=self.limit)

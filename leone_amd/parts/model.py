@@ -7,7 +7,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from .. import ops
-from ..weights.loader import MATRIX, TensorSpec
+from ..weights.loader import MATRIX, VECTOR, TensorSpec
 from .base import BLOCKS, NORMS, POSITIONS, PartSpec, flatten_needs, nest_views
 from .context import CacheView, StepContext
 
@@ -19,11 +19,17 @@ class LayerRun:
     ``layer`` indexes ``ModelSpec.layers`` (a layer may be named more than
     once).  ``cache`` is the cache slot the run works on; two runs that name the
     same slot share it, and only runs with ``writes`` put new keys, values or
-    state there.
+    state there.  ``borrow`` (for a layer whose cache need is a dict): name -> the
+    cache slot of another run whose storage of that name this run reads without
+    writing, while everything else it keeps is its own.
     """
     layer: int
     cache: Optional[int]
     writes: bool = True
+    borrow: Optional[Dict[str, int]] = None
+
+    def __hash__(self):
+        return hash((self.layer, self.cache, self.writes, tuple(sorted((self.borrow or {}).items()))))
 
 
 @dataclass
@@ -41,6 +47,9 @@ class ModelSpec:
     embedding_scale: Optional[float] = None         # the stream starts as table row * scale
     logit_cap: Optional[float] = None               # logits = cap * tanh(logits / cap)
     position_table: Optional[str] = None            # tensor name [max_positions, hidden]: a learned vector a position, added to the token's
+    # One tensor name for every scheduled run (or None): behind run i the stream becomes the sum over j <= i + 1 of
+    # weight_i[j] * X_j, with X_0 the embedding's output and X_(j+1) run j's own result; weight_i has i + 2 elements.
+    depth_weights: Optional[Sequence[str]] = None
 
 
 def default_schedule(n_layers: int) -> List[LayerRun]:
@@ -63,6 +72,9 @@ class DecoderModel:
         for run in self.schedule:
             if not 0 <= run.layer < len(self.layers):
                 raise ValueError(f"schedule names layer {run.layer}, the model has {len(self.layers)}")
+        if spec.depth_weights is not None and len(spec.depth_weights) != len(self.schedule):
+            raise ValueError(f"{len(spec.depth_weights)} depth weights for {len(self.schedule)} layer runs")
+        self.depth_weights: Optional[List[torch.Tensor]] = None
         self.embedding: Optional[torch.Tensor] = None
         self.position_table: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
@@ -81,6 +93,8 @@ class DecoderModel:
             specs.append(TensorSpec(self.spec.position_table, (self.spec.max_positions, self.spec.hidden_size), MATRIX))
         for layer in self.layers:
             specs += layer.tensor_specs()
+        for at, name in enumerate(self.spec.depth_weights or ()):
+            specs.append(TensorSpec(name, (at + 2,), VECTOR))
         specs += self.final_norm.tensor_specs()
         if self.spec.head is not None:
             specs.append(TensorSpec(self.spec.head, (self.spec.vocab_size, self.spec.hidden_size), MATRIX))
@@ -94,6 +108,8 @@ class DecoderModel:
         self.head = tensors.pop(self.spec.head).contiguous() if self.spec.head is not None else self.embedding
         for layer in self.layers:
             layer.bind(tensors)
+        if self.spec.depth_weights is not None:
+            self.depth_weights = [tensors.pop(name).contiguous() for name in self.spec.depth_weights]
         self.final_norm.bind(tensors)
         for position in self.positions.values():
             position.prepare(self.spec.max_positions, self.device)
@@ -201,9 +217,12 @@ class DecoderModel:
             if run.cache is None:
                 raise ValueError(f"layer {run.layer} needs a cache but its run names none")
             for path, leaf in leaves:
-                key = (run.cache,) + path if isinstance(need, dict) else run.cache
+                lent = self._lender(run, need, path)
+                key = ((run.cache if lent is None else lent,) + path) if isinstance(need, dict) else run.cache
                 if key in needs and needs[key] != leaf:
                     raise ValueError(f"cache slot {key} is shared by layers with different needs")
+                if lent is not None and key not in needs:
+                    raise ValueError(f"layer {run.layer} borrows cache slot {key}, which no earlier run keeps")
                 needs[key] = leaf
             writers[run.cache] = writers.get(run.cache, 0) + (1 if run.writes else 0)
         for slot, count in writers.items():
@@ -212,22 +231,45 @@ class DecoderModel:
         return needs
 
     @staticmethod
+    def _lender(run: LayerRun, need, path) -> Optional[int]:
+        """The slot of the run that lends this run the storage at ``path`` of its needs, or None if it is its own."""
+        if run.borrow and isinstance(need, dict) and path and path[0] in run.borrow:
+            return run.borrow[path[0]]
+        return None
+
+    @staticmethod
     def _cache_of(run: LayerRun, layer, caches: Dict[object, CacheView]):
         """What a run's layer receives as its cache: the view of the run's slot, or, for a layer with several
         needs, the views in the shape of its needs."""
         if run.cache is None:
             return None
 
-        def view(key):
+        def view(key, writes=run.writes):
             found = caches.get(key)
-            if found is not None and found.writes != run.writes:
-                found = type(found)(**{**found.__dict__, "writes": run.writes})
+            if found is not None and found.writes != writes:
+                found = type(found)(**{**found.__dict__, "writes": writes})
             return found
 
         need = layer.cache_need()
         if isinstance(need, dict):
-            return nest_views(need, (run.cache,), view)
+            def lookup(key):
+                lent = DecoderModel._lender(run, need, key[1:])
+                return view(key, run.writes) if lent is None else view((lent,) + key[1:], False)
+            return nest_views(need, (run.cache,), lookup)
         return view(run.cache)
+
+    def _mix_depth(self, x: torch.Tensor, pending, history: torch.Tensor, at: int):
+        """x + pending is run ``at``'s own result: it is kept, and the stream becomes the weighted sum of all results
+        so far, in one kernel."""
+        scale = 1.0
+        if isinstance(pending, ops.PreparedRows):
+            pending = None
+        elif isinstance(pending, ops.ScaledDelta):
+            pending, scale = pending.rows, pending.scale
+        elif isinstance(pending, ops.NormedDelta):
+            pending = pending.materialize()
+        ops.depth_mix(x, pending, scale, history, at + 2, self.depth_weights[at])
+        return None
 
     # ---- forward ---------------------------------------------------------------
     def forward(self, tokens: torch.Tensor, step: StepContext, caches: Dict[int, CacheView]) -> Optional[torch.Tensor]:
@@ -237,6 +279,11 @@ class DecoderModel:
         x = ops.embed(self.embedding, tokens, scale=self.spec.embedding_scale or 1.0,
                       position_table=self.position_table, positions=step.positions)
         pending = None
+        history = None
+        if self.depth_weights is not None:
+            # every run's own result is kept for the step: the stream behind a run is mixed from all of them
+            history = torch.empty((len(self.schedule) + 1, *x.shape), dtype=torch.float32, device=x.device)
+            history[0].copy_(x)
         for at, run in enumerate(self.schedule):
             layer = self.layers[run.layer]
             cache = self._cache_of(run, layer, caches)
@@ -247,12 +294,16 @@ class DecoderModel:
                 pending = layer.forward(x, pending, step, cache, next_norm=next_norm)
             else:
                 pending = layer.forward(x, pending, step, cache)
+            if history is not None:
+                pending = self._mix_depth(x, pending, history, at)
         if step.want_rows is None or step.want_rows.numel() == 0:
             if pending is not None:
                 pass  # nothing reads the last delta when no logits are wanted
             return None
         if isinstance(pending, ops.PreparedRows):
             pending = None                    # prepared for a norm that never ran: the stream is up to date
+        if isinstance(pending, ops.ScaledDelta) and not hasattr(self.final_norm, "gain"):
+            pending = pending.materialize()
         if hasattr(self.final_norm, "lazy"):
             y = self.final_norm.lazy(x, pending, self.dtype, rows=step.want_rows)
         else:

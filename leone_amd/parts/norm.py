@@ -35,6 +35,9 @@ class RmsNorm(Part):
                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         if isinstance(delta, ops.PreparedRows):
             delta = None                      # the product that made it has added into the stream already
+        if isinstance(delta, ops.ScaledDelta):
+            # a sublayer's result that enters the stream times a factor: sum and norm in one kernel
+            return ops.residual_norm(x, delta.rows, delta.scale, self.gain, self.eps, out_dtype, rows)
         if isinstance(delta, ops.NormedDelta):
             behind = delta.norm
             if isinstance(behind, RmsNorm) and behind.gain.dtype == self.gain.dtype:
@@ -106,6 +109,8 @@ class LayerNorm(Part):
         if isinstance(delta, ops.PreparedRows):
             delta = None
         delta_norm = None
+        if isinstance(delta, ops.ScaledDelta):
+            delta = delta.materialize()
         if isinstance(delta, ops.NormedDelta):
             behind = delta.norm
             if isinstance(behind, LayerNorm) and behind.gain.dtype == self.gain.dtype:

@@ -230,6 +230,61 @@ class ChannelDeltaMixer(Part):
         return ops.linear(y, self.w_o, out_dtype=torch.float32)
 
 
+@MIXERS.register("hgrn2")
+class GatedMemoryMixer(Part):
+    """Linear attention whose forget gate also decides what is written (HGRN2): there is no key projection.
+
+    q = silu(Wq h) (``heads`` of ``dim``), v = Wv h (``heads`` of ``vdim``), forget gate per head and key channel
+    f = lower + (1 - lower) * sigmoid(Wf h + f_bias) with a stored lower bound.  Per head S' = diag(f) S + (1 - f) v^T
+    (f on the rows of S that belong to q's channels), o = S'^T q; each head's o over its root mean square times ``norm``
+    (size vdim, shared by the heads), then Wo.  The state is float32 and starts at zero.
+
+    Parameters: ``hidden``, ``heads``, ``dim``, ``vdim``, ``eps`` and tensor names ``q``, ``f``, ``f_bias``, ``lower``,
+    ``v``, ``norm``, ``o``.
+    """
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, **_):
+        p = spec.params
+        self.hidden, self.heads, self.dim, self.vdim = (int(p[k]) for k in ("hidden", "heads", "dim", "vdim"))
+        self.eps = float(p["eps"])
+        _check_dim("hgrn2", self.dim)
+        self.names = {k: p[k] for k in ("q", "f", "f_bias", "lower", "v", "norm", "o")}
+        qk = self.heads * self.dim
+        self.columns = {"q": 0, "f": qk, "v": 2 * qk}
+        self.w_in = self.w_o = self.norm = self.f_bias = self.lower = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        n, qk, vv = self.names, self.heads * self.dim, self.heads * self.vdim
+        return [TensorSpec(n["q"], (qk, self.hidden), MATRIX), TensorSpec(n["f"], (qk, self.hidden), MATRIX),
+                TensorSpec(n["f_bias"], (qk,), VECTOR), TensorSpec(n["lower"], (qk,), VECTOR),
+                TensorSpec(n["v"], (vv, self.hidden), MATRIX), TensorSpec(n["norm"], (self.vdim,), VECTOR),
+                TensorSpec(n["o"], (self.hidden, vv), MATRIX)]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.w_in = torch.cat([tensors.pop(self.names[k]) for k in ("q", "f", "v")], dim=0).contiguous()
+        self.w_o = tensors.pop(self.names["o"]).contiguous()
+        self.norm = tensors.pop(self.names["norm"]).contiguous()
+        self.f_bias = tensors.pop(self.names["f_bias"]).contiguous()
+        self.lower = tensors.pop(self.names["lower"]).contiguous()
+        if self.f_bias.dtype != self.lower.dtype:
+            self.f_bias, self.lower = self.f_bias.float(), self.lower.float()
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_in, self.w_o]
+
+    def cache_need(self) -> StateNeed:
+        return StateNeed((self.heads, self.dim * self.vdim), torch.float32)
+
+    def forward(self, h: torch.Tensor, step: StepContext, cache) -> torch.Tensor:
+        proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
+        o = ops.gated_scan(proj, self.columns, self.f_bias, self.lower, cache.state, step, self.heads, self.dim, self.vdim,
+                           q_activation="silu", write_state=cache.writes)
+        y = ops.head_norm_gate(o, self.heads, self.vdim, self.eps, step.dtype, gain=self.norm)
+        return ops.linear(y, self.w_o, out_dtype=torch.float32)
+
+
 @MIXERS.register("parallel")
 class ParallelMixer(Part):
     """Several mixers side by side on the same input: each result is divided by its root mean square over the
