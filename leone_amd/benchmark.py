@@ -391,7 +391,33 @@ def zukinex_shape(width: int, layers: int, vocab: int, context: int) -> dict:
             "max_positions": max(4096, context + 64), "layers": listed}
 
 
-DESIGN_SHAPES = {"pamevik": pamevik_shape, "zukinex": zukinex_shape}
+def fosulix_shape(width: int, layers: int, vocab: int, context: int) -> dict:
+    """Fosulix at layer sizes that resemble published models of its kinds: latent attention with heads of 128 plain and
+    64 rotated elements, values of 128, a query latent of 3/8 width and a key/value latent of 512, a window of 1,024,
+    frequencies stretched eightfold; of four layers the second reads the first's latents and the third is a matrix
+    memory with heads of 128 x 128; every layer with 32 experts of 3/8 width of which four are chosen (eight groups of
+    which four stay open): 1.5 x width of feed-forward a token."""
+    rot = {"dims": 64, "base": 10000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+
+    def latent(kv_from=None):
+        m = {"heads": width // 128, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": 3 * width // 8, "kv_rank": 512,
+             "scale": 192 ** -0.5, "rot": rot, "mask": {"size": 1024}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "latent_attention", "mixer": m}
+    routed = {"kind": "moe", "expert": {"ff": 3 * width // 8, "limit": 7.0},
+              "router": {"experts": 32, "top": 4, "scale": 2.5, "groups": {"count": 8, "keep": 4}}}
+    listed = []
+    for i in range(layers):
+        kind = i % 4
+        entry = ({"type": "hgrn2", "mixer": {"heads": width // 128, "dim": 128, "vdim": 128}} if kind == 2
+                 else latent(i - 1 if kind == 1 else None))
+        listed.append({**entry, "mlp": routed})
+    return {"architecture": "Fosulix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "embedding": {"scale": 1.0}, "canon": {"taps": 4}, "max_positions": max(4096, context + 64), "layers": listed}
+
+
+DESIGN_SHAPES = {"pamevik": pamevik_shape, "zukinex": zukinex_shape, "fosulix": fosulix_shape}
 
 
 def state_bytes_per_request(model) -> int:

@@ -20,8 +20,14 @@
 //                     cached vector is read once for all of the workgroup's heads), lanes split the elements; the
 //                     waves' partial results are merged in a fixed order.
 //
-// The cache of one layer: [page][token in page][rank + rot] in the engine's type.  Norms, angles, scores, softmax and
-// all sums are float.
+//   latent_attention_cores  the same on the matrix cores (bfloat16): a workgroup takes 16 (row, head) pairs, its four
+//                     waves take 32-key tiles in turn; S^T = K Q^T and O^T += V^T P^T with v_mfma_f32_16x16x32_bf16,
+//                     both operands straight from the cache in 16-byte runs.
+//
+// The cache of one layer holds a token's vector twice, each time in the order one of the two products reads it:
+// as a key, [page][element / 8][token in page][8] over the rank + rot elements (filled up to a multiple of 8), and
+// as a value, [page][token in page / 8][element][8] over the first `rank` elements.  Norms, angles, scores, softmax
+// and all sums are float.
 #include "common.h"
 #include "leone_hip.h"
 
@@ -47,7 +53,8 @@ latent_prepare_kernel(const float* __restrict__ proj, long stride, int q_off, in
                       int kv_off, int rank, int rot, AnyVec kv_gain, float eps, const float* __restrict__ cos_table,
                       const float* __restrict__ sin_table, int rot_half, int table_positions,
                       const int* __restrict__ positions, const int* __restrict__ row_entry,
-                      const int* __restrict__ block_table, int max_blocks, int page_tokens, T* __restrict__ pool) {
+                      const int* __restrict__ block_table, int max_blocks, int page_tokens, T* __restrict__ k_pool,
+                      T* __restrict__ v_pool) {
     __shared__ float scratch[kLatWaves];
     const int row = blockIdx.x;
     const float* base = proj + static_cast<long>(row) * stride;
@@ -62,55 +69,83 @@ latent_prepare_kernel(const float* __restrict__ proj, long stride, int q_off, in
     const int pos = positions[row];
     const int page = block_table[static_cast<long>(row_entry[row]) * max_blocks + pos / page_tokens];
     if (page < 0) return;                                       // no page mapped: nothing is written outside the pool
-    T* to = pool + (static_cast<long>(page) * page_tokens + pos % page_tokens) * (rank + rot);
+    const int tok = pos % page_tokens, runs = (rank + rot + 7) / 8;
+    T* as_key = k_pool + static_cast<long>(page) * runs * page_tokens * 8;
+    T* as_value = v_pool + (static_cast<long>(page) * (page_tokens / 8) + tok / 8) * rank * 8 + tok % 8;
+    auto put = [&](int e, T v) { as_key[(static_cast<long>(e / 8) * page_tokens + tok) * 8 + e % 8] = v; };
     const float* kv = base + kv_off;
     float ss = 0.f;
     for (int c = threadIdx.x; c < rank; c += kLatThreads) ss = fmaf(kv[c], kv[c], ss);
     const float inv = 1.0f / sqrtf(block_sum<kLatThreads>(ss, scratch) / static_cast<float>(rank) + eps);
-    for (int c = threadIdx.x; c < rank; c += kLatThreads) to[c] = from_float<T>(kv[c] * inv * load_any(kv_gain, c));
+    for (int c = threadIdx.x; c < rank; c += kLatThreads) {
+        const T v = from_float<T>(kv[c] * inv * load_any(kv_gain, c));
+        put(c, v);
+        as_value[static_cast<long>(c) * 8] = v;
+    }
     const int at = min(pos, table_positions - 1);
     const float* cos_row = cos_table ? cos_table + static_cast<long>(at) * rot_half : nullptr;
     const float* sin_row = cos_table ? sin_table + static_cast<long>(at) * rot_half : nullptr;
     for (int c = threadIdx.x; c < rot; c += kLatThreads)
-        to[rank + c] = from_float<T>(rotated_adjacent(kv + rank, c, cos_row, sin_row, rot_half));
+        put(rank + c, from_float<T>(rotated_adjacent(kv + rank, c, cos_row, sin_row, rot_half)));
+    for (int c = rank + rot + threadIdx.x; c < runs * 8; c += kLatThreads) put(c, from_float<T>(0.f));
 }
 
 constexpr int kHpRows = 8;
+constexpr int kHpCols = 64;          // output columns a workgroup takes; its four waves split the inner elements
 
-// x: [rows] rows of x_row_stride floats or TX, head h's `inner` elements at h * x_head_stride; w: [heads][inner][outer];
-// y: rows of y_row_stride, head h's results at h * y_head_stride.  A thread owns one output column for 8 rows.
+// x: [rows] rows of x_row_stride floats or TX, head h's `inner` elements at h * x_head_stride; w: [heads][inner][outer]
+// (null: only the tail is handed on); y: rows of y_row_stride, head h's results at h * y_head_stride.  A workgroup takes
+// 8 rows, one head and 64 columns; a lane owns a column, a wave a quarter of the inner elements; the waves' sums are
+// added in their order.
 template <typename TX, typename TW, typename TY>
 __global__ void __launch_bounds__(kLatThreads)
 head_product_kernel(const TX* __restrict__ x, long x_row_stride, long x_head_stride, const TW* __restrict__ w,
                     TY* __restrict__ y, long y_row_stride, long y_head_stride, int rows, int inner, int outer, int tail,
                     const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot_half,
                     int table_positions, const int* __restrict__ positions) {
-    extern __shared__ __align__(16) float hp_lds[];            // [kHpRows][inner + tail]
+    extern __shared__ __align__(16) float hp_lds[];            // [kHpRows][inner + tail], then [waves][kHpRows][kHpCols]
     const int head = blockIdx.y, row0 = blockIdx.x * kHpRows;
     const int here = min(kHpRows, rows - row0);
     const int width = inner + tail;
+    float* partial = hp_lds + kHpRows * width;
     for (int idx = threadIdx.x; idx < kHpRows * width; idx += kLatThreads) {
         const int r = idx / width, k = idx % width;
         hp_lds[idx] = r < here ? to_float(x[(row0 + r) * x_row_stride + head * x_head_stride + k]) : 0.f;
     }
     __syncthreads();
-    const TW* wh = w + static_cast<long>(head) * inner * outer;
-    for (int n = threadIdx.x; n < outer; n += kLatThreads) {
+    if (w) {
+        const int lane = threadIdx.x % kWave, part = threadIdx.x / kWave;
+        const int n = blockIdx.z * kHpCols + lane;
+        const int share = (inner + kLatWaves - 1) / kLatWaves;
+        const int k0 = part * share, k1 = min(inner, k0 + share);
         float acc[kHpRows];
 #pragma unroll
         for (int r = 0; r < kHpRows; ++r) acc[r] = 0.f;
-        for (int k = 0; k < inner; ++k) {
-            const float wv = to_float(wh[static_cast<long>(k) * outer + n]);
+        if (n < outer) {
+            const TW* wh = w + static_cast<long>(head) * inner * outer + n;
+#pragma unroll 4
+            for (int k = k0; k < k1; ++k) {
+                const float wv = to_float(wh[static_cast<long>(k) * outer]);
 #pragma unroll
-            for (int r = 0; r < kHpRows; ++r) acc[r] = fmaf(hp_lds[r * width + k], wv, acc[r]);
+                for (int r = 0; r < kHpRows; ++r) acc[r] = fmaf(hp_lds[r * width + k], wv, acc[r]);
+            }
         }
 #pragma unroll
-        for (int r = 0; r < kHpRows; ++r)
-            if (r < here) y[(row0 + r) * y_row_stride + head * y_head_stride + n] = from_float<TY>(acc[r]);
+        for (int r = 0; r < kHpRows; ++r) partial[(part * kHpRows + r) * kHpCols + lane] = acc[r];
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < here * kHpCols; idx += kLatThreads) {
+            const int r = idx / kHpCols, col = idx % kHpCols;
+            if (blockIdx.z * kHpCols + col >= outer) continue;
+            float sum = 0.f;
+#pragma unroll
+            for (int p = 0; p < kLatWaves; ++p) sum += partial[(p * kHpRows + r) * kHpCols + col];
+            y[(row0 + r) * y_row_stride + head * y_head_stride + blockIdx.z * kHpCols + col] = from_float<TY>(sum);
+        }
     }
+    if (blockIdx.z != 0) return;
     for (int idx = threadIdx.x; idx < here * tail; idx += kLatThreads) {
         const int r = idx / tail, c = idx % tail;
-        const int at = min(positions[row0 + r], table_positions - 1);
+        const int at = cos_table ? min(positions[row0 + r], table_positions - 1) : 0;
         const float* cos_row = cos_table ? cos_table + static_cast<long>(at) * rot_half : nullptr;
         const float* sin_row = cos_table ? sin_table + static_cast<long>(at) * rot_half : nullptr;
         y[(row0 + r) * y_row_stride + head * y_head_stride + outer + c] =
@@ -157,12 +192,12 @@ latent_attention_kernel(const float* __restrict__ q, float* __restrict__ out, co
             for (int h = 0; h < kHeads; ++h) l[h] = __builtin_nanf("");
             continue;
         }
-        const T* kr = pool + (static_cast<long>(page) * page_tokens + j % page_tokens) * width;
+        const T* kr = pool + (static_cast<long>(page) * ((width + 7) / 8) * page_tokens + j % page_tokens) * 8;
         float kv[kChunks];
 #pragma unroll
         for (int i = 0; i < kChunks; ++i) {
             const int d = lane + i * kWave;
-            kv[i] = d < width ? to_float(kr[d]) : 0.f;
+            kv[i] = d < width ? to_float(kr[static_cast<long>(d / 8) * page_tokens * 8 + d % 8]) : 0.f;
         }
 #pragma unroll
         for (int h = 0; h < kHeads; ++h) {
@@ -237,6 +272,211 @@ static int pick_latent_attention(const float* q, float* out, const void* pool, c
 #undef LEONE_LATENT
 }
 
+
+// ---- the same on the matrix cores ------------------------------------------------------------------------------
+//
+// Operand layouts of v_mfma_f32_16x16x32_bf16 (lane l, c = l % 16, g = l / 16): A: row c, k-slots 8g .. 8g+7; B: column
+// c, k-slots 8g .. 8g+7; C/D: column c, rows 4g .. 4g+3.  A workgroup's 16 columns are 16 consecutive (row, head)
+// pairs of the step; they may belong to several requests (single decoded tokens of a model with few heads), which
+// are then taken one after the other with the other requests' columns masked.  For S^T the two 16-key halves of a
+// 32-key tile are laid out so that lane (g, c) ends up with the scores of keys 8g .. 8g+7 of the tile: the k-slots it
+// supplies as P^T to the second product.  Each wave keeps a running maximum and sum per column; the waves' partial
+// results are merged in shared memory in the waves' order.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 lat_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float lat_floatx4;
+
+constexpr int kCoreTile = 32;        // keys of a tile
+
+__device__ inline lat_bf16x8 lat_load8(const bf16_t* p) {
+    return __builtin_bit_cast(lat_bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+__device__ inline lat_bf16x8 lat_zero8() {
+    return __builtin_bit_cast(lat_bf16x8, uint4{0u, 0u, 0u, 0u});
+}
+
+// kSteps * 32 >= rank + rot, kDT * 16 >= rank; `steps` and `dts` are the counts in use.
+template <int kSteps, int kDT>
+__global__ void __launch_bounds__(kLatThreads)
+latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ out, const bf16_t* __restrict__ k_pool,
+                              const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
+                              const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
+                              int total, int heads, int rank, int width, int page_tokens, float to_log2, int window) {
+    extern __shared__ __align__(16) float lc_lds[];               // [16][rank + 4] sums, then [waves][16] maxima, [waves][16] sums
+    const int pitch = rank + 4;
+    float* sm_acc = lc_lds;
+    float* sm_m = lc_lds + 16 * pitch;
+    float* sm_l = sm_m + kLatWaves * 16;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int c = lane % 16, g = lane / 16;
+    const int steps = width / 32, dts = rank / 16;
+    const long pair = static_cast<long>(blockIdx.x) * 16 + c;     // this lane's column: (row, head) pair of the step
+    const bool valid = pair < total;
+    const int row = valid ? static_cast<int>(pair / heads) : 0;
+    const int pos = valid ? positions[row] : -1;
+    const int entry = valid ? row_entry[row] : -1;
+    const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+
+    lat_bf16x8 qreg[kSteps];
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s)
+        qreg[s] = (valid && s < steps) ? lat_load8(q + pair * width + 32 * s + 8 * g) : lat_zero8();
+    lat_floatx4 acc[kDT];
+#pragma unroll
+    for (int dt = 0; dt < kDT; ++dt) acc[dt] = lat_floatx4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    bool unmapped = false;
+    const long key_page = static_cast<long>(width / 8) * page_tokens * 8;      // elements of a page, as keys
+    const long value_page = static_cast<long>(page_tokens / 8) * rank * 8;      // and as values
+
+    int at = 0;                                                   // first column of the request that is walked next
+    while (at < 16) {
+        const int walked = __shfl(entry, at, kWave);              // lanes 0..15 are the columns with g = 0
+        if (walked < 0) break;                                    // columns beyond the step's last pair
+        const bool mine = valid && entry == walked;
+        at += __popcll(__ballot(mine) & 0xffffull);               // a request's columns stand side by side
+        int hi = mine ? pos : -1, lo = mine ? first : 0x7fffffff;
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) {
+            hi = max(hi, __shfl_xor(hi, off, kWave));
+            lo = min(lo, __shfl_xor(lo, off, kWave));
+        }
+        const int* table = block_table + static_cast<long>(walked) * max_blocks;
+        for (int t = lo / kCoreTile + wave; t <= hi / kCoreTile; t += kLatWaves) {
+            const int key0 = t * kCoreTile;
+            const int page = table[key0 / page_tokens];
+            const int tok0 = key0 % page_tokens;
+            if (page < 0) {                                       // a key in reach without a page: say so in the result
+                unmapped = true;
+                continue;
+            }
+            const bool inner = key0 >= lo && key0 + kCoreTile - 1 <= hi;     // every key of the tile belongs to the request's range
+            // ---- S^T = K Q^T for the two 16-key halves ----
+            const int ka = 8 * (c >> 2) + (c & 3);                // this lane's key of the first half; the second's is 4 further
+            const bf16_t* kp = k_pool + page * key_page + static_cast<long>(tok0 + ka) * 8;
+            lat_floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < kSteps; ++s) {
+                if (s < steps) {
+                    const bf16_t* from = kp + static_cast<long>(4 * s + g) * page_tokens * 8;
+                    lat_bf16x8 xa = lat_load8(from), xb = lat_load8(from + 32);
+                    if (!inner) {                                 // what lies outside the range may hold anything
+                        if (key0 + ka < lo || key0 + ka > hi) xa = lat_zero8();
+                        if (key0 + ka + 4 < lo || key0 + ka + 4 > hi) xb = lat_zero8();
+                    }
+                    sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, qreg[s], sa, 0, 0, 0);
+                    sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb, qreg[s], sb, 0, 0, 0);
+                }
+            }
+            // lane (g, c) holds, for column c, the scores of keys key0 + 8g + j, j = 0 .. 7
+            const int run0 = key0 + 8 * g;
+            float sc[8], tile_max = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int key = run0 + j;
+                const float raw = j < 4 ? sa[j & 3] : sb[j & 3];
+                sc[j] = (mine && key >= first && key <= pos) ? raw * to_log2 : -INFINITY;
+                tile_max = fmaxf(tile_max, sc[j]);
+            }
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+            const float m_new = fmaxf(m_run, tile_max);
+            const bool none = m_new == -INFINITY;                 // a column that has seen no key yet
+            const float alpha = none ? 1.f : __builtin_amdgcn_exp2f(m_run - m_new);
+            float psum = 0.f;
+            lat_bf16x8 pt;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                pt[j] = static_cast<__bf16>(none ? 0.f : __builtin_amdgcn_exp2f(sc[j] - m_new));
+                psum += static_cast<float>(pt[j]);
+            }
+            psum += __shfl_xor(psum, 16, kWave);
+            psum += __shfl_xor(psum, 32, kWave);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+            // ---- O^T += V^T P^T ----
+            const bf16_t* vp = v_pool + page * value_page + (static_cast<long>((tok0 + 8 * g) / 8) * rank + c) * 8;
+            unsigned keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+            if (!inner) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int e0 = run0 + 2 * i, e1 = e0 + 1;
+                    keep[i] = ((e0 >= lo && e0 <= hi) ? 0x0000ffffu : 0u) | ((e1 >= lo && e1 <= hi) ? 0xffff0000u : 0u);
+                }
+            }
+#pragma unroll
+            for (int dt = 0; dt < kDT; ++dt) {
+                if (dt < dts) {
+                    uint4 raw = *reinterpret_cast<const uint4*>(vp + static_cast<long>(16 * dt) * 8);
+                    if (!inner) {
+                        raw.x &= keep[0];
+                        raw.y &= keep[1];
+                        raw.z &= keep[2];
+                        raw.w &= keep[3];
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[dt][r] *= alpha;
+                    acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lat_bf16x8, raw), pt, acc[dt], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // ---- merge the four waves, in their order ----
+    if (__any(unmapped)) l_run = __builtin_nanf("");
+    if (g == 0) {
+        sm_m[wave * 16 + c] = m_run;
+        sm_l[wave * 16 + c] = l_run;
+    }
+    __syncthreads();
+    float top = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kLatWaves; ++w) top = fmaxf(top, sm_m[w * 16 + c]);
+    float denom = 0.f;
+#pragma unroll
+    for (int w = 0; w < kLatWaves; ++w) {
+        const float mw = sm_m[w * 16 + c];
+        denom += sm_l[w * 16 + c] * (mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - top));
+    }
+    const float weight = (m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - top)) / denom;
+    for (int w = 0; w < kLatWaves; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int dt = 0; dt < kDT; ++dt) {
+                if (dt < dts) {
+                    float4* to = reinterpret_cast<float4*>(sm_acc + c * pitch + 16 * dt + 4 * g);
+                    float4 sum = w == 0 ? float4{0.f, 0.f, 0.f, 0.f} : *to;
+                    sum.x += acc[dt][0] * weight;
+                    sum.y += acc[dt][1] * weight;
+                    sum.z += acc[dt][2] * weight;
+                    sum.w += acc[dt][3] * weight;
+                    *to = sum;
+                }
+            }
+        }
+        __syncthreads();
+    }
+    const long pair0 = static_cast<long>(blockIdx.x) * 16;
+    for (int i = threadIdx.x; i < 16 * rank; i += kLatThreads) {
+        const int col = i / rank, e = i % rank;
+        if (pair0 + col < total) out[(pair0 + col) * rank + e] = sm_acc[col * pitch + e];
+    }
+}
+
+template <int kSteps, int kDT>
+static int launch_latent_cores(const void* q, float* out, const void* k_pool, const void* v_pool, const int* positions,
+                               const int* row_entry, const int* block_table, int max_blocks, int rows, int heads, int rank,
+                               int rot, int page_tokens, float scale, int window, hipStream_t stream) {
+    const long total = static_cast<long>(rows) * heads;
+    const size_t shared = (static_cast<size_t>(16) * (rank + 4) + 2 * kLatWaves * 16) * sizeof(float);
+    LEONE_REQUIRE(shared <= 64 * 1024 && (total + 15) / 16 <= 0x7fffffffL, "latent_attention_cores: %ld pairs, a latent of %d", total, rank);
+    latent_attention_cores_kernel<kSteps, kDT><<<static_cast<unsigned>((total + 15) / 16), kLatThreads, shared, stream>>>(
+        static_cast<const bf16_t*>(q), out, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), positions,
+        row_entry, block_table, max_blocks, static_cast<int>(total), heads, rank, rank + rot, page_tokens,
+        scale * 1.4426950408889634f, window);
+    LEONE_LAUNCH_CHECK("latent_attention_cores");
+    return 0;
+}
+
 }  // namespace leone
 
 using namespace leone;
@@ -246,19 +486,19 @@ extern "C" int leone_latent_max_width() { return 18 * kWave; }
 // proj float32 [rows, stride].  q_off >= 0: the query latent's q_rank columns from there, RMS-normed times q_gain, go
 // to q_out [rows, q_rank] of `dtype`.  kv_off >= 0: the key/value latent's `rank` columns and the shared key part's
 // `rot` columns from there go, normed (times kv_gain) and rotated (tables [table_positions, rot_half], pairs (2i, 2i+1)
-// of the part's first 2 * rot_half elements), into pool [pages, page_tokens, rank + rot] of `dtype`.
+// of the part's first 2 * rot_half elements), into the two pools of `dtype` (the layouts at the top).
 extern "C" int leone_latent_prepare(const float* proj, long stride, int rows, int q_off, int q_rank, const void* q_gain,
                                     void* q_out, int kv_off, int rank, int rot, const void* kv_gain, int gain_dtype, float eps,
                                     const float* cos_table, const float* sin_table, int rot_half, int table_positions,
                                     const int* positions, const int* row_entry, const int* block_table, int max_blocks,
-                                    int page_tokens, void* pool, int dtype, hipStream_t stream) {
+                                    int page_tokens, void* k_pool, void* v_pool, int dtype, hipStream_t stream) {
     LEONE_REQUIRE(dtype == kF32 || dtype == kBF16, "latent_prepare: unknown element type %d", dtype);
     LEONE_REQUIRE(gain_dtype == kF32 || gain_dtype == kBF16, "latent_prepare: unknown type of the gains");
     LEONE_REQUIRE(proj && rows > 0 && eps > 0.f && (q_off >= 0 || kv_off >= 0), "latent_prepare: null pointer, no rows or nothing to do");
     LEONE_REQUIRE(q_off < 0 || (q_gain && q_out && q_rank > 0 && stride >= q_off + q_rank), "latent_prepare: the query latent does not fit rows of %ld", stride);
     if (kv_off >= 0) {
-        LEONE_REQUIRE(kv_gain && pool && positions && row_entry && block_table, "latent_prepare: a cache write needs a pool, positions, a row map and a block table");
-        LEONE_REQUIRE(rank > 0 && rot >= 0 && stride >= kv_off + rank + rot && max_blocks > 0 && page_tokens > 0,
+        LEONE_REQUIRE(kv_gain && k_pool && v_pool && positions && row_entry && block_table, "latent_prepare: a cache write needs both pools, positions, a row map and a block table");
+        LEONE_REQUIRE(rank > 0 && rot >= 0 && stride >= kv_off + rank + rot && max_blocks > 0 && page_tokens > 0 && page_tokens % 8 == 0,
                       "latent_prepare: a latent of %d + %d does not fit rows of %ld", rank, rot, stride);
         LEONE_REQUIRE((cos_table == nullptr) == (sin_table == nullptr) && (!cos_table || (rot_half > 0 && 2 * rot_half <= rot && table_positions > 0)),
                       "latent_prepare: tables for %d pairs of a part of %d", rot_half, rot);
@@ -267,12 +507,12 @@ extern "C" int leone_latent_prepare(const float* proj, long stride, int rows, in
         latent_prepare_kernel<float><<<rows, kLatThreads, 0, stream>>>(
             proj, stride, q_off, q_rank, AnyVec{q_gain, gain_dtype}, static_cast<float*>(q_out), kv_off, rank, rot,
             AnyVec{kv_gain, gain_dtype}, eps, cos_table, sin_table, cos_table ? rot_half : 0, table_positions, positions, row_entry,
-            block_table, max_blocks, page_tokens, static_cast<float*>(pool));
+            block_table, max_blocks, page_tokens, static_cast<float*>(k_pool), static_cast<float*>(v_pool));
     else
         latent_prepare_kernel<bf16_t><<<rows, kLatThreads, 0, stream>>>(
             proj, stride, q_off, q_rank, AnyVec{q_gain, gain_dtype}, static_cast<bf16_t*>(q_out), kv_off, rank, rot,
             AnyVec{kv_gain, gain_dtype}, eps, cos_table, sin_table, cos_table ? rot_half : 0, table_positions, positions, row_entry,
-            block_table, max_blocks, page_tokens, static_cast<bf16_t*>(pool));
+            block_table, max_blocks, page_tokens, static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool));
     LEONE_LAUNCH_CHECK("latent_prepare");
     return 0;
 }
@@ -284,16 +524,16 @@ extern "C" int leone_head_product(const float* x, long x_row_stride, long x_head
                                   int tail, const float* cos_table, const float* sin_table, int rot_half, int table_positions,
                                   const int* positions, hipStream_t stream) {
     LEONE_REQUIRE((w_dtype == kF32 || w_dtype == kBF16) && (y_dtype == kF32 || y_dtype == kBF16), "head_product: unknown element type");
-    LEONE_REQUIRE(x && w && y && rows > 0 && heads > 0 && heads <= 65535 && inner > 0 && outer > 0 && tail >= 0,
+    LEONE_REQUIRE(x && y && rows > 0 && heads > 0 && heads <= 65535 && inner > 0 && outer > 0 && tail >= 0 && (w || tail > 0),
                   "head_product: null pointer or empty sizes");
     LEONE_REQUIRE(x_head_stride >= inner + tail && x_row_stride >= (heads - 1) * x_head_stride + inner + tail &&
                   y_head_stride >= outer + tail && y_row_stride >= (heads - 1) * y_head_stride + outer + tail,
                   "head_product: rows too short for %d heads of %d + %d in, %d + %d out", heads, inner, tail, outer, tail);
     LEONE_REQUIRE((cos_table == nullptr) == (sin_table == nullptr) && (!cos_table || (rot_half > 0 && 2 * rot_half <= tail && table_positions > 0 && positions)),
                   "head_product: tables for %d pairs of a tail of %d", rot_half, tail);
-    const size_t shared = static_cast<size_t>(kHpRows) * (inner + tail) * sizeof(float);
-    LEONE_REQUIRE(shared <= 64 * 1024, "head_product: %d + %d elements a head are too many", inner, tail);
-    const dim3 grid(ceil_div(rows, kHpRows), heads);
+    const size_t shared = (static_cast<size_t>(kHpRows) * (inner + tail) + kLatWaves * kHpRows * kHpCols) * sizeof(float);
+    LEONE_REQUIRE(shared <= 64 * 1024 && ceil_div(outer, kHpCols) <= 65535, "head_product: %d + %d elements a head are too many", inner, tail);
+    const dim3 grid(ceil_div(rows, kHpRows), heads, w ? ceil_div(outer, kHpCols) : 1);
     const int half = cos_table ? rot_half : 0;
 #define LEONE_HP(TW, TY)                                                                                               \
     head_product_kernel<float, TW, TY><<<grid, kLatThreads, shared, stream>>>(                                         \
@@ -313,7 +553,7 @@ extern "C" int leone_head_product(const float* x, long x_row_stride, long x_head
 
 // q float32 [rows, heads, rank + rot] (up-projection already taken to the query's side, shared key part rotated);
 // out float32 [rows, heads, rank]: sum_j p_j c_j over the keys j of the row's request with pos - window < j <= pos
-// (window 0: all j <= pos); pool [pages, page_tokens, rank + rot] of `dtype`.
+// (window 0: all j <= pos); pool: the keys' form of the cache, of `dtype`.
 extern "C" int leone_latent_attention(const float* q, float* out, const void* pool, int dtype, const int* positions,
                                       const int* row_entry, const int* block_table, int max_blocks, int rows, int heads,
                                       int rank, int rot, int page_tokens, float scale, int window, hipStream_t stream) {
@@ -328,4 +568,29 @@ extern "C" int leone_latent_attention(const float* q, float* out, const void* po
                                             page_tokens, scale, window, stream);
     return pick_latent_attention<bf16_t>(q, out, pool, positions, row_entry, block_table, max_blocks, rows, heads, rank, rot,
                                          page_tokens, scale, window, stream);
+}
+
+// The same on the matrix cores: bfloat16 queries [rows, heads, rank + rot] and both forms of the cache; rank + rot a
+// multiple of 32 up to leone_latent_cores_max_width(), rank a multiple of 16, pages of a multiple of 32 tokens.
+extern "C" int leone_latent_cores_max_width() { return 576; }
+
+extern "C" int leone_latent_attention_cores(const void* q, float* out, const void* k_pool, const void* v_pool, const int* positions,
+                                            const int* row_entry, const int* block_table, int max_blocks, int rows, int heads,
+                                            int rank, int rot, int page_tokens, float scale, int window, hipStream_t stream) {
+    LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table, "latent_attention_cores: null pointer");
+    LEONE_REQUIRE(rows > 0 && heads > 0 && rank > 0 && rot >= 0 && (rank + rot) % 32 == 0 && rank % 16 == 0 &&
+                  rank + rot <= leone_latent_cores_max_width(),
+                  "latent_attention_cores: rows %d, %d heads, a latent of %d + %d", rows, heads, rank, rot);
+    LEONE_REQUIRE(page_tokens > 0 && page_tokens % 32 == 0 && max_blocks > 0 && window >= 0 && scale > 0.f,
+                  "latent_attention_cores: page_tokens %d, max_blocks %d, window %d", page_tokens, max_blocks, window);
+    LEONE_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(k_pool) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(v_pool) % 16 == 0, "latent_attention_cores: operands must lie on 16-byte borders");
+    const int width = rank + rot;
+#define LEONE_LATENT_CORES(S, D)                                                                                          \
+    return launch_latent_cores<S, D>(q, out, k_pool, v_pool, positions, row_entry, block_table, max_blocks, rows, heads, rank, \
+                                     rot, page_tokens, scale, window, stream)
+    if (width <= 128) LEONE_LATENT_CORES(4, 8);
+    if (width <= 256) LEONE_LATENT_CORES(8, 16);
+    LEONE_LATENT_CORES(18, 32);
+#undef LEONE_LATENT_CORES
 }

@@ -319,7 +319,8 @@ int leone_latent_max_width();
 int leone_latent_prepare(const float* proj, long stride, int rows, int q_off, int q_rank, const void* q_gain, void* q_out,
                          int kv_off, int rank, int rot, const void* kv_gain, int gain_dtype, float eps, const float* cos_table,
                          const float* sin_table, int rot_half, int table_positions, const int* positions, const int* row_entry,
-                         const int* block_table, int max_blocks, int page_tokens, void* pool, int dtype, hipStream_t stream);
+                         const int* block_table, int max_blocks, int page_tokens, void* k_pool, void* v_pool, int dtype,
+                         hipStream_t stream);
 int leone_head_product(const float* x, long x_row_stride, long x_head_stride, const void* w, int w_dtype, void* y, int y_dtype,
                        long y_row_stride, long y_head_stride, int rows, int heads, int inner, int outer, int tail,
                        const float* cos_table, const float* sin_table, int rot_half, int table_positions, const int* positions,
@@ -327,6 +328,10 @@ int leone_head_product(const float* x, long x_row_stride, long x_head_stride, co
 int leone_latent_attention(const float* q, float* out, const void* pool, int dtype, const int* positions, const int* row_entry,
                            const int* block_table, int max_blocks, int rows, int heads, int rank, int rot, int page_tokens,
                            float scale, int window, hipStream_t stream);
+int leone_latent_cores_max_width();
+int leone_latent_attention_cores(const void* q, float* out, const void* k_pool, const void* v_pool, const int* positions,
+                                 const int* row_entry, const int* block_table, int max_blocks, int rows, int heads, int rank,
+                                 int rot, int page_tokens, float scale, int window, hipStream_t stream);
 // Residual sums with a factor; the stream as a weighted sum of every earlier layer's result (see depth.hip).
 int leone_residual_norm(float* x, const float* delta, int planes, long plane, float scale, const void* gain, int gain_dtype,
                         float eps, void* y, int y_dtype, const int* rows, int n_rows, int hidden, hipStream_t stream);

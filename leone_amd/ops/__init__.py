@@ -1676,12 +1676,13 @@ def latent_prepare(proj: torch.Tensor, out_dtype: torch.dtype, eps: float, *, q_
                    kv_gain: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
                    sin: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
                    row_entry: Optional[torch.Tensor] = None, block_table: Optional[torch.Tensor] = None,
-                   pool: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                   k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """From the float32 down-projections ``proj [rows, width]``: the query latent (``q_rank`` columns from
     ``q_column``) RMS-normed times ``q_gain`` comes back in ``out_dtype``; the key/value latent (``rank`` columns from
     ``kv_column``) RMS-normed times ``kv_gain`` and the ``rot`` columns behind it, rotated in neighbouring pairs by the
-    row's position, are written into ``pool [pages, page_tokens, rank + rot]`` at the row's place.  Either half may be
-    left out."""
+    row's position, are written at the row's place into the cache: as a key into ``k_pool [pages, ceil((rank + rot) / 8),
+    page_tokens, 8]`` and the latent once more as a value into ``v_pool [pages, page_tokens / 8, rank, 8]``.  Either half
+    may be left out."""
     rows, width = proj.shape
     q_out = torch.empty((rows, q_rank), dtype=out_dtype, device=proj.device) if q_column is not None else None
     gains = [g for g in (q_gain, kv_gain) if g is not None]
@@ -1689,12 +1690,10 @@ def latent_prepare(proj: torch.Tensor, out_dtype: torch.dtype, eps: float, *, q_
         raise KernelError("latent_prepare: the gains must come in one type")
     page_tokens = max_blocks = 0
     if kv_column is not None:
-        if pool is None or pool.dim() != 3 or pool.shape[2] != rank + rot or pool.dtype != out_dtype:
-            raise KernelError(f"latent_prepare: the pool must be {out_dtype} [pages, page_tokens, {rank + rot}], found "
-                              f"{None if pool is None else (pool.dtype, tuple(pool.shape))}")
+        page_tokens = _latent_pools("latent_prepare", k_pool, v_pool, rank, rot, out_dtype)
         if block_table is None or positions is None or row_entry is None:
             raise KernelError("latent_prepare: a cache write needs positions, a row map and a block table")
-        page_tokens, max_blocks = pool.shape[1], block_table.shape[1]
+        max_blocks = block_table.shape[1]
     cos_at, sin_at, pairs, table_positions = _rotation_tables("latent_prepare", rot, cos, sin)
     call("leone_latent_prepare", _dev(proj, "projection", torch.float32), width, rows,
          -1 if q_column is None else int(q_column), int(q_rank), _dev(q_gain, "query gain", None, (q_rank,)) if q_column is not None else 0,
@@ -1704,8 +1703,24 @@ def latent_prepare(proj: torch.Tensor, out_dtype: torch.dtype, eps: float, *, q_
          _dev(positions, "positions", torch.int32, (rows,)) if kv_column is not None else 0,
          _dev(row_entry, "row map", torch.int32, (rows,)) if kv_column is not None else 0,
          _dev(block_table, "block table", torch.int32) if kv_column is not None else 0, max_blocks, page_tokens,
-         _dev(pool, "latent pool") if kv_column is not None else 0, _CODES[out_dtype], _stream())
+         _dev(k_pool, "latent keys") if kv_column is not None else 0, _dev(v_pool, "latent values") if kv_column is not None else 0,
+         _CODES[out_dtype], _stream())
     return q_out
+
+
+def _latent_pools(what: str, k_pool, v_pool, rank: int, rot: int, dtype) -> int:
+    """Checks the two forms of a latent cache against each other and the sizes; returns the tokens a page holds."""
+    runs = -(-(rank + rot) // 8)
+    if k_pool is None or v_pool is None or k_pool.dim() != 4 or v_pool.dim() != 4 or k_pool.shape[1] != runs or k_pool.shape[3] != 8 \
+            or tuple(v_pool.shape) != (k_pool.shape[0], k_pool.shape[2] // 8, rank, 8) or k_pool.shape[2] % 8 \
+            or k_pool.dtype != v_pool.dtype or (dtype is not None and k_pool.dtype != dtype):
+        raise KernelError(f"{what}: the cache must be [pages, {runs}, page_tokens, 8] and [pages, page_tokens / 8, {rank}, 8] of one "
+                          f"type, found {None if k_pool is None else (k_pool.dtype, tuple(k_pool.shape))} and "
+                          f"{None if v_pool is None else (v_pool.dtype, tuple(v_pool.shape))}")
+    return k_pool.shape[2]
+
+
+HEAD_PRODUCT_LIBRARY_ROWS = 128      # from here on a bfloat16 product a head goes to the library's batched product
 
 
 def head_product(x: torch.Tensor, weight: torch.Tensor, heads: int, out_dtype: torch.dtype, *, tail: int = 0,
@@ -1714,36 +1729,69 @@ def head_product(x: torch.Tensor, weight: torch.Tensor, heads: int, out_dtype: t
     """A product a head: ``x`` float32 ``[rows, heads * (inner + tail)]``, ``weight`` ``[heads, inner, outer]`` ->
     ``[rows, heads * (outer + tail)]`` in ``out_dtype`` with y[r, h, :outer] = x[r, h, :inner] weight[h].  The ``tail``
     elements behind a head's inner ones are handed on behind its outer ones, rotated in neighbouring pairs by the
-    row's position if tables come."""
+    row's position if tables come.  Many rows of a bfloat16 model go through the library's batched product (the rows
+    as two bfloat16 parts, float accumulation); the kernel then hands on the tails alone."""
     rows = x.shape[0]
     if weight.dim() != 3 or weight.shape[0] != heads or x.dim() != 2 or x.shape[1] != heads * (weight.shape[1] + tail):
         raise KernelError(f"head_product: rows {tuple(x.shape)} against {tuple(weight.shape)} for {heads} heads with a tail of {tail}")
     inner, outer = weight.shape[1], weight.shape[2]
     out = torch.empty((rows, heads * (outer + tail)), dtype=out_dtype, device=x.device)
     cos_at, sin_at, pairs, table_positions = _rotation_tables("head_product", tail, cos, sin)
-    call("leone_head_product", _dev(x, "head rows", torch.float32), x.shape[1], inner + tail, _dev(weight, "head matrices"),
-         _code(weight, "head matrices"), _dev(out, "head results"), _CODES[out_dtype], out.shape[1], outer + tail, rows, heads,
+    library = weight.dtype == torch.bfloat16 and rows >= HEAD_PRODUCT_LIBRARY_ROWS and inner % 8 == 0 and outer % 8 == 0
+    if library:
+        with profile.span(profile.LIBRARY_PRODUCT, weight):
+            # the float32 rows as a sum of two bfloat16 parts, so that the result is that of the kernel for few rows
+            # (float32 rows against bfloat16 matrices) up to the order of the sums
+            part = x.view(rows, heads, inner + tail)[:, :, :inner]
+            high = part.to(torch.bfloat16)
+            low = (part - high).to(torch.bfloat16)
+            y = torch.bmm(high.transpose(0, 1), weight, out_dtype=torch.float32)
+            y += torch.bmm(low.transpose(0, 1), weight, out_dtype=torch.float32)
+            out.view(rows, heads, outer + tail)[:, :, :outer].copy_(y.transpose(0, 1))
+        if not tail:
+            return out
+    call("leone_head_product", _dev(x, "head rows", torch.float32), x.shape[1], inner + tail,
+         0 if library else _dev(weight, "head matrices"), _code(weight, "head matrices"), _dev(out, "head results"),
+         _CODES[out_dtype], out.shape[1], outer + tail, rows, heads,
          inner, outer, int(tail), cos_at, sin_at, pairs, table_positions,
          _dev(positions, "positions", torch.int32, (rows,)) if cos is not None else 0, _stream())
     return out
 
 
-def latent_attention(q: torch.Tensor, pool: torch.Tensor, positions: torch.Tensor, row_entry: torch.Tensor,
-                     block_table: torch.Tensor, heads: int, rank: int, rot: int, scale: float, window: int = 0) -> torch.Tensor:
-    """Softmax attention over a cache of latents shared by the heads: ``q`` float32 ``[rows, heads * (rank + rot)]`` (the
-    keys' up-projection already on the query's side, see ``head_product``), ``pool`` ``[pages, page_tokens, rank + rot]``;
+def latent_cores_supported(dtype: torch.dtype, rank: int, rot: int, page_tokens: int) -> bool:
+    """Whether the matrix-core kernel takes a latent cache of these sizes; otherwise the kernel for any size does."""
+    return (dtype == torch.bfloat16 and (rank + rot) % 32 == 0 and rank % 16 == 0 and page_tokens % 32 == 0
+            and rank + rot <= library().leone_latent_cores_max_width())
+
+
+def latent_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
+                     row_entry: torch.Tensor, block_table: torch.Tensor, heads: int, rank: int, rot: int, scale: float,
+                     window: int = 0) -> torch.Tensor:
+    """Softmax attention over a cache of latents shared by the heads: ``q`` ``[rows, heads * (rank + rot)]`` (the keys'
+    up-projection already on the query's side, see ``head_product``), the cache in its two forms (``latent_prepare``);
     a row sees the latents of its request at positions pos - window < j <= pos (``window`` 0: all).  Returns float32
-    ``[rows, heads * rank]``: every head's weighted sum of the latents' first ``rank`` elements."""
+    ``[rows, heads * rank]``: every head's weighted sum of the latents.  bfloat16 queries go to the matrix-core kernel
+    (``latent_cores_supported``), float32 queries to the kernel for any size and type of cache."""
     rows = q.shape[0]
-    if pool.dim() != 3 or pool.shape[2] != rank + rot or q.shape[1] != heads * (rank + rot):
-        raise KernelError(f"latent_attention: queries {tuple(q.shape)} and pool {tuple(pool.shape)} do not fit {heads} heads of {rank} + {rot}")
+    page_tokens = _latent_pools("latent_attention", k_pool, v_pool, rank, rot, None)
+    if q.shape[1] != heads * (rank + rot):
+        raise KernelError(f"latent_attention: queries {tuple(q.shape)} do not fit {heads} heads of {rank} + {rot}")
+    out = torch.empty((rows, heads * rank), dtype=torch.float32, device=q.device)
+    if q.dtype == torch.bfloat16:
+        if not latent_cores_supported(k_pool.dtype, rank, rot, page_tokens):
+            raise KernelError(f"latent_attention: bfloat16 queries are for the matrix-core kernel, which does not take a "
+                              f"{k_pool.dtype} cache of {rank} + {rot} in pages of {page_tokens}")
+        call("leone_latent_attention_cores", _dev(q, "latent queries", torch.bfloat16), _dev(out, "latent sums"),
+             _dev(k_pool, "latent keys"), _dev(v_pool, "latent values"), _dev(positions, "positions", torch.int32, (rows,)),
+             _dev(row_entry, "row map", torch.int32, (rows,)), _dev(block_table, "block table", torch.int32),
+             block_table.shape[1], rows, heads, int(rank), int(rot), page_tokens, float(scale), int(window), _stream())
+        return out
     if rank + rot > library().leone_latent_max_width():
         raise KernelError(f"latent_attention: a latent of {rank} + {rot} elements, the kernel takes {library().leone_latent_max_width()}")
-    out = torch.empty((rows, heads * rank), dtype=torch.float32, device=q.device)
-    call("leone_latent_attention", _dev(q, "latent queries", torch.float32), _dev(out, "latent sums"), _dev(pool, "latent pool"),
-         _code(pool, "latent pool"), _dev(positions, "positions", torch.int32, (rows,)),
+    call("leone_latent_attention", _dev(q, "latent queries", torch.float32), _dev(out, "latent sums"), _dev(k_pool, "latent keys"),
+         _code(k_pool, "latent keys"), _dev(positions, "positions", torch.int32, (rows,)),
          _dev(row_entry, "row map", torch.int32, (rows,)), _dev(block_table, "block table", torch.int32), block_table.shape[1],
-         rows, heads, int(rank), int(rot), pool.shape[1], float(scale), int(window), _stream())
+         rows, heads, int(rank), int(rot), page_tokens, float(scale), int(window), _stream())
     return out
 
 

@@ -87,7 +87,8 @@ _PROTOTYPES = {
                          ctypes.c_long, P, P, c_int, c_int, c_int, P],
     "leone_gated_chain": [P, c_int, P, ctypes.c_long, P, P, ctypes.c_long, c_int, c_int, c_int, c_int, P],
     "leone_latent_prepare": [P, ctypes.c_long, c_int, c_int, c_int, P, P, c_int, c_int, c_int, P, c_int, c_float, P, P, c_int, c_int,
-                             P, P, P, c_int, c_int, P, c_int, P],
+                             P, P, P, c_int, c_int, P, P, c_int, P],
+    "leone_latent_attention_cores": [P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "leone_head_product": [P, ctypes.c_long, ctypes.c_long, P, c_int, P, c_int, ctypes.c_long, ctypes.c_long, c_int, c_int, c_int,
                            c_int, c_int, P, P, c_int, c_int, P, P],
     "leone_latent_attention": [P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
@@ -135,6 +136,8 @@ def library() -> ctypes.CDLL:
             lib.leone_moe_tile_pairs.argtypes = []
             lib.leone_latent_max_width.restype = c_int
             lib.leone_latent_max_width.argtypes = []
+            lib.leone_latent_cores_max_width.restype = c_int
+            lib.leone_latent_cores_max_width.argtypes = []
             lib.leone_route_max_outputs.restype = c_int
             lib.leone_route_max_outputs.argtypes = []
             lib.leone_library_product_available.restype = c_int

@@ -63,6 +63,7 @@ OPERATIONS = {
     "leone_latent_prepare": "latent norm rope kv",
     "leone_head_product": "head product",
     "leone_latent_attention": "attention",
+    "leone_latent_attention_cores": "attention",
     "leone_residual_norm": "norm",
     "leone_depth_mix": "depth mix",
 }

@@ -15,7 +15,8 @@ from .position import rotation_of
 
 @dataclass
 class LatentCacheView(CacheView):
-    pool: torch.Tensor = None          # [pages, page_tokens, rank + rot]
+    k_pool: torch.Tensor = None        # [pages, ceil((rank + rot) / 8), page_tokens, 8]: a token's vector as a key
+    v_pool: torch.Tensor = None        # [pages, page_tokens / 8, rank, 8]: its latent once more, as a value
     block_table: torch.Tensor = None   # int32 [entries, max_blocks] of the layer's group
     page_tokens: int = 0
 
@@ -23,7 +24,9 @@ class LatentCacheView(CacheView):
 @dataclass(frozen=True)
 class LatentNeed:
     """A mixer that caches, per token, one latent of ``rank`` elements and a rotated key part of ``rot`` elements that
-    all its heads share: ``[pages, page_tokens, rank + rot]`` in the engine's type."""
+    all its heads share, in the engine's type.  The vector is kept twice, packed in runs of 8 in the order each of
+    attention's two products reads it: as a key ``[pages, ceil((rank + rot) / 8), page_tokens, 8]`` and, its latent
+    alone, as a value ``[pages, page_tokens / 8, rank, 8]``."""
     rank: int
     rot: int
     window: Optional[int] = None        # only the last `window` positions are ever read
@@ -36,16 +39,21 @@ class LatentNeed:
         return self
 
     def allocate(self, pages: int, page_tokens: int, dtype: torch.dtype, device):
-        return torch.zeros((pages, page_tokens, self.rank + self.rot), dtype=dtype, device=device)
+        if page_tokens % 8:
+            raise ValueError(f"the cache packs runs of 8 tokens: page_tokens {page_tokens} must be a multiple of 8")
+        return (torch.zeros((pages, -(-(self.rank + self.rot) // 8), page_tokens, 8), dtype=dtype, device=device),
+                torch.zeros((pages, page_tokens // 8, self.rank, 8), dtype=dtype, device=device))
 
     def view(self, storage, block_table, page_tokens: int):
-        return LatentCacheView(writes=True, pool=storage, block_table=block_table, page_tokens=page_tokens)
+        return LatentCacheView(writes=True, k_pool=storage[0], v_pool=storage[1], block_table=block_table,
+                               page_tokens=page_tokens)
 
     def poison(self, storage, index: torch.Tensor) -> None:
-        storage.index_fill_(0, index, float("nan"))
+        for pool in storage:
+            pool.index_fill_(0, index, float("nan"))
 
     def bytes_per_token(self, element_size: int) -> int:
-        return (self.rank + self.rot) * element_size
+        return (-(-(self.rank + self.rot) // 8) * 8 + self.rank) * element_size
 
 
 @MIXERS.register("latent_attention")
@@ -132,14 +140,16 @@ class LatentAttention(Part):
         c_q = ops.latent_prepare(down, step.dtype, self.eps, q_column=0, q_rank=self.q_rank, q_gain=self.q_gain,
                                  kv_column=self.q_rank if writes else None, rank=self.kv_rank, rot=self.rot_dim,
                                  kv_gain=self.kv_gain, cos=rotation.cos, sin=rotation.sin, positions=step.positions,
-                                 row_entry=step.row_entry, block_table=cache.block_table, pool=cache.pool)
+                                 row_entry=step.row_entry, block_table=cache.block_table, k_pool=cache.k_pool,
+                                 v_pool=cache.v_pool)
         q = ops.linear(c_q, self.w_uq, out_dtype=torch.float32)
         if q.dim() == 3:
             q = q.sum(dim=0)
-        # W_uk on the query's side; the rotated query part behind it
-        q = ops.head_product(q, self.w_uk, self.heads, torch.float32, tail=self.rot_dim, cos=rotation.cos, sin=rotation.sin,
-                             positions=step.positions)
-        mixed = ops.latent_attention(q, cache.pool, step.positions, step.row_entry, cache.block_table, self.heads,
-                                     self.kv_rank, self.rot_dim, self.scale, int(self.window or 0))
+        # W_uk on the query's side; the rotated query part behind it.  The matrix-core kernel reads its queries in bfloat16.
+        cores = ops.latent_cores_supported(step.dtype, self.kv_rank, self.rot_dim, cache.page_tokens)
+        q = ops.head_product(q, self.w_uk, self.heads, step.dtype if cores else torch.float32, tail=self.rot_dim,
+                             cos=rotation.cos, sin=rotation.sin, positions=step.positions)
+        mixed = ops.latent_attention(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry, cache.block_table,
+                                     self.heads, self.kv_rank, self.rot_dim, self.scale, int(self.window or 0))
         values = ops.head_product(mixed, self.w_uv, self.heads, step.dtype)
         return ops.linear(values, self.w_o, out_dtype=torch.float32)

@@ -94,7 +94,7 @@ class DecoderModel:
         for layer in self.layers:
             specs += layer.tensor_specs()
         for at, name in enumerate(self.spec.depth_weights or ()):
-            specs.append(TensorSpec(name, (at + 2,), VECTOR))
+            specs.append(TensorSpec(name, (at + 2,), VECTOR, init=("normal", 1.0 / (at + 2), 0.02)))     # about an average
         specs += self.final_norm.tensor_specs()
         if self.spec.head is not None:
             specs.append(TensorSpec(self.spec.head, (self.spec.vocab_size, self.spec.hidden_size), MATRIX))

@@ -258,7 +258,8 @@ class GatedMemoryMixer(Part):
     def tensor_specs(self) -> List[TensorSpec]:
         n, qk, vv = self.names, self.heads * self.dim, self.heads * self.vdim
         return [TensorSpec(n["q"], (qk, self.hidden), MATRIX), TensorSpec(n["f"], (qk, self.hidden), MATRIX),
-                TensorSpec(n["f_bias"], (qk,), VECTOR), TensorSpec(n["lower"], (qk,), VECTOR),
+                TensorSpec(n["f_bias"], (qk,), VECTOR, init=("normal", 0.0, 1.0)),
+                TensorSpec(n["lower"], (qk,), VECTOR, init=("uniform", 0.0, 1.0)),      # a lower bound of a gate in (0, 1)
                 TensorSpec(n["v"], (vv, self.hidden), MATRIX), TensorSpec(n["norm"], (self.vdim,), VECTOR),
                 TensorSpec(n["o"], (self.hidden, vv), MATRIX)]
 

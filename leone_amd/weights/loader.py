@@ -32,6 +32,9 @@ class TensorSpec:
     shape: tuple
     role: str = MATRIX
     optional: bool = False
+    # how random weights of this tensor are drawn where the role's rule would give values the part cannot take:
+    # ("uniform", low, high) or ("normal", mean, deviation); None: the role's rule
+    init: tuple = None
 
 
 class WeightsError(ValueError):

@@ -1,7 +1,8 @@
 """Random weights from a configuration and a seed.
 
 Matrices and embedding tables are drawn from N(0, 0.02), norm gains from
-1 + N(0, 0.02).  Each tensor has its own generator keyed by (seed, tensor name),
+1 + N(0, 0.02); a tensor whose spec names a rule of its own (``TensorSpec.init``)
+follows that.  Each tensor has its own generator keyed by (seed, tensor name),
 so a tensor's values do not depend on which other tensors exist or in which
 order they are made.  ``write_model_dir`` writes a model folder (config.json,
 model.safetensors) that loads like any other; ``device_tensors`` makes the same
@@ -31,9 +32,14 @@ def host_tensor(spec: TensorSpec, seed: int, dtype: torch.dtype) -> torch.Tensor
     rng = np.random.Generator(np.random.Philox(key=_key(seed, spec.name)))
     if spec.role == INT_TABLE:
         raise ValueError(f"{spec.name}: no rule for random integer tables")
-    values = rng.standard_normal(size=spec.shape, dtype=np.float32) * np.float32(STD)
-    if spec.role == VECTOR:
-        values += np.float32(1.0)
+    if spec.init is not None and spec.init[0] == "uniform":
+        values = (rng.random(size=spec.shape, dtype=np.float32) * np.float32(spec.init[2] - spec.init[1]) + np.float32(spec.init[1]))
+    elif spec.init is not None:
+        values = rng.standard_normal(size=spec.shape, dtype=np.float32) * np.float32(spec.init[2]) + np.float32(spec.init[1])
+    else:
+        values = rng.standard_normal(size=spec.shape, dtype=np.float32) * np.float32(STD)
+        if spec.role == VECTOR:
+            values += np.float32(1.0)
     return torch.from_numpy(values).to(dtype)
 
 
@@ -46,9 +52,14 @@ def device_tensors(specs: Iterable[TensorSpec], seed: int, dtype: torch.dtype, d
     for spec in specs:
         gen = torch.Generator(device=device)
         gen.manual_seed((int(seed) * 1000003 + zlib.crc32(spec.name.encode("utf-8"))) & 0x7FFFFFFFFFFFFFFF)
-        t = torch.randn(spec.shape, generator=gen, device=device, dtype=torch.float32) * STD
-        if spec.role == VECTOR:
-            t += 1.0
+        if spec.init is not None and spec.init[0] == "uniform":
+            t = torch.rand(spec.shape, generator=gen, device=device, dtype=torch.float32) * (spec.init[2] - spec.init[1]) + spec.init[1]
+        elif spec.init is not None:
+            t = torch.randn(spec.shape, generator=gen, device=device, dtype=torch.float32) * spec.init[2] + spec.init[1]
+        else:
+            t = torch.randn(spec.shape, generator=gen, device=device, dtype=torch.float32) * STD
+            if spec.role == VECTOR:
+                t += 1.0
         out[spec.name] = t.to(dtype)
         del t
     return out

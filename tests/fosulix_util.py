@@ -73,6 +73,18 @@ SMALL = {
         layer(latent(4, 32, 64, 32, 96, 128, base=1000.0, scaling=(2.0, 16, 4.0, 1.0), mask=5), None),
         layer(memory(2, 64, 32), moe(4, 4, 32, scale=0.25)),
     ], mult=0.7, embed_scale=11.0, taps=5),
+    # latents of 128, 256 and 576 elements in multiples of 32 with parts in multiples of 16: in bfloat16 and pages of 32
+    # tokens attention goes to the matrix-core kernel, with 3, 4 and 16 heads (16 heads fill a tile of 16 columns, fewer
+    # heads put several rows, in steps of single tokens several requests, into one).  Its mixtures take all their
+    # experts, so that no rounded router input changes a choice at an early position and, through attention and memory,
+    # every later position with it: what differs from the plain results in bfloat16 is then attention's rounding.
+    "D": config(128, 300, [
+        layer(latent(4, 16, 32, 16, 32, 96, base=1000.0, scaling=(8.0, 64, 32.0, 1.0), mask=40), moe(4, 4, 32, groups=(2, 2), scale=1.5)),
+        layer(latent(16, 8, 32, 8, 64, 96, base=1000.0, scaling=(8.0, 64, 32.0, 1.0), mask=70, kv_from=0), None),
+        layer(memory(2, 32, 32), moe(3, 3, 32)),
+        layer(latent(3, 32, 32, 24, 48, 224, base=500.0), moe(2, 2, 48, limit=1.0)),
+        layer(latent(2, 16, 64, 16, 32, 512, base=10000.0, mask=33), None),
+    ], mult=0.5, embed_scale=6.0, taps=3),
 }
 
 

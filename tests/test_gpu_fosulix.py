@@ -28,7 +28,8 @@ F = torch.float64
 # by an expert's whole output: so the median must keep the bound and at most one position in twelve may be beyond
 # five times it.  A fault (a wrong key, a window off by one, a lost state) moves most positions.
 TOLERANCE = {"float32": 3e-5, "bfloat16": 3e-2}
-LENGTHS = {"A": [1, 2, 37, 130, 64, 9], "B": [70, 3, 150, 33, 81], "C": [90, 17, 65, 2, 48]}
+LENGTHS = {"A": [1, 2, 37, 130, 64, 9], "B": [70, 3, 150, 33, 81], "C": [90, 17, 65, 2, 48], "D": [100, 5, 140, 31, 66, 1]}
+PAGE_TOKENS = {"A": 16, "B": 16, "C": 16, "D": 32}
 
 
 def widened(weights):
@@ -43,7 +44,9 @@ def cases(tmp_path_factory):
         key = (name, dtype_name)
         if key not in cache:
             raw = fu.SMALL[name]
-            weights = fu.make_weights(raw, 17 + len(cache), DTYPES[dtype_name], sharpen=2.5 if dtype_name == "float32" else 1.0)
+            # D's latents of hundreds of elements give scores of tens as they are: sharper ones only magnify float rounding
+            sharpen = 1.0 if dtype_name != "float32" else 1.2 if name == "D" else 2.5
+            weights = fu.make_weights(raw, 17 + len(cache), DTYPES[dtype_name], sharpen=sharpen)
             folder = fu.write_dir(str(tmp_path_factory.mktemp(f"fosulix_{name}_{dtype_name}")), raw, weights)
             gen = np.random.default_rng(5 + len(cache))
             requests = {f"r{i}": gen.integers(0, raw["vocab"], size=n).tolist() for i, n in enumerate(LENGTHS[name])}
@@ -109,7 +112,12 @@ def test_engine_agrees_with_plain_however_the_work_is_cut(cases, name, dtype_nam
     position."""
     folder, requests, expected = cases(name, dtype_name)
     steps = SCHEDULES[schedule](requests)
-    engine = make_engine(folder, dtype_name, max_tokens=schedules.max_live_tokens(steps, 16), poison_freed=True)
+    page = PAGE_TOKENS[name]
+    engine = make_engine(folder, dtype_name, max_tokens=schedules.max_live_tokens(steps, page), page_tokens=page, poison_freed=True)
+    if name == "D":
+        from leone_amd import ops
+        assert all(ops.latent_cores_supported(engine.model.dtype, layer.mixer.kv_rank, layer.mixer.rot_dim, page) == (dtype_name == "bfloat16")
+                   for layer in engine.model.layers if hasattr(layer.mixer, "kv_rank"))
     outputs = run_steps(engine, steps)
     worst = compare(steps, outputs, expected, dtype_name, f"{name} {dtype_name} {schedule}")
     print(f"{name} {dtype_name} {schedule}: worst relative error {worst:.2e}")
@@ -140,7 +148,8 @@ def test_pages_and_slots_that_held_another_request(cases, dtype_name):
         outputs = run_steps(engine, steps)
         compare(steps, outputs, {rid: expected[rid]}, dtype_name, f"page reuse {rid}")
         for storage in engine.pools.paged.values():
-            storage.fill_(float("nan"))
+            for pool in storage:
+                pool.fill_(float("nan"))
         for storage in engine.pools.state.values():
             storage.fill_(float("nan"))
 
@@ -297,35 +306,41 @@ LATENTS = [
      "rot": {"dims": 16, "base": 1000.0, "scaling": {"factor": 2.0, "original": 16, "fast": 4.0, "slow": 2.0}}, "mask": {"size": 1}},
     {"heads": 6, "dim": 64, "rot_dim": 32, "vdim": 64, "q_rank": 96, "kv_rank": 320, "scale": 0.1,
      "rot": {"dims": 32, "base": 10000.0}, "mask": {"size": 32}},
+    {"heads": 16, "dim": 32, "rot_dim": 64, "vdim": 32, "q_rank": 64, "kv_rank": 512, "scale": 0.1,
+     "rot": {"dims": 64, "base": 10000.0}, "mask": {"size": 45}},
+    {"heads": 5, "dim": 16, "rot_dim": 16, "vdim": 24, "q_rank": 32, "kv_rank": 48, "scale": 0.2, "rot": {"dims": 16, "base": 100.0}},
 ]
 
 
+@pytest.mark.parametrize("page_tokens", [16, 32])
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 @pytest.mark.parametrize("m", LATENTS, ids=lambda m: f"{m['heads']}x{m['dim']}+{m['rot_dim']}r{m['kv_rank']}")
-def test_latent_attention_alone_in_cuts_of_every_size(m, dtype_name):
+def test_latent_attention_alone_in_cuts_of_every_size(m, dtype_name, page_tokens):
     """Two sequences side by side, fed in steps of 0 to 40 rows each, state slots and pages interleaved and filled
-    with NaN beforehand: one head and several, latents of 24 to 320 elements, a window of one key (itself), of a
-    page and a bit, of two pages, and none."""
+    with NaN beforehand: one head and several, latents of 24 to 512 elements, a window of one key (itself), of a
+    page and a bit, of two pages, and none.  In bfloat16 with pages of 32 tokens the sizes that fit go to the
+    matrix-core kernel."""
     dtype = DTYPES[dtype_name]
     part, w, width = latent_case(dtype, m, seed=m["kv_rank"])
     gen = torch.Generator().manual_seed(3)
     hs = [torch.randn(63, width, generator=gen).to(dtype), torch.randn(66, width, generator=gen).to(dtype)]
-    got = run_mixer_in_cuts(part, hs, CUTS, dtype)
+    got = run_mixer_in_cuts(part, hs, CUTS, dtype, page_tokens)
     for s in (0, 1):
         want = plain_latent(hs[s].to(F), m, w)
         err = fu.relative_error(got[s].numpy(), want.numpy())
         assert err.max() <= (2e-5 if dtype_name == "float32" else 3e-2), (s, int(err.argmax()), float(err.max()))
 
 
+@pytest.mark.parametrize("page_tokens", [16, 32])
 @pytest.mark.parametrize("window", [None, 40, 64])
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
-def test_latent_attention_finds_planted_keys(dtype_name, window):
+def test_latent_attention_finds_planted_keys(dtype_name, window, page_tokens):
     """Keys that answer one query each are planted far back, on both sides of page borders (pages of 16), and at the
     last position a window still holds; a decoy stands one position outside the window of a query, with a value of its
     own, and must not be seen.  Queries come in a prompt's portion and as single decoded tokens.  The plain part of the
     query meets the latent through W_uk; the weights here make that the identity on the first elements."""
     dtype = DTYPES[dtype_name]
-    width, heads, dim, rot, vdim, qr, kr = 48, 2, 12, 4, 16, 24, 24
+    width, heads, dim, rot, vdim, qr, kr = 48, 2, 12, 32, 16, 24, 32      # a latent of 32 + 32: with pages of 32 the matrix cores
     m = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "q_rank": qr, "kv_rank": kr, "scale": 1.0,
          "rot": {"dims": rot, "base": 10.0}}
     if window:
@@ -368,7 +383,7 @@ def test_latent_attention_finds_planted_keys(dtype_name, window):
     hs = hs.to(dtype)
     want = plain_latent(hs.to(F), m, w)
     cuts = [(270, 1), (10, 1)] + [(1, 1)] * 20
-    got = run_mixer_in_cuts(part, [hs, hs[:22]], cuts, dtype)[0]
+    got = run_mixer_in_cuts(part, [hs, hs[:22]], cuts, dtype, page_tokens)[0]
     err = fu.relative_error(got.numpy(), want.numpy())
     tol = 2e-5 if dtype_name == "float32" else 3e-2
     asked = list(pairs.values())

@@ -250,20 +250,20 @@ def views_of(need, slots=3, pages=40, page_tokens=16, dtype=torch.float32):
     return made
 
 
-def nested(need, made, table):
+def nested(need, made, table, page_tokens=16):
     from leone_amd.parts.base import nest_views
     def view(path):
         kind, leaf, storage = made[path]
-        return leaf.view(storage, table, 16) if kind == "paged" else leaf.view(storage)
+        return leaf.view(storage, table, page_tokens) if kind == "paged" else leaf.view(storage)
     return nest_views(need, (), view)
 
 
-def run_mixer_in_cuts(mixer, hs, cuts, dtype):
+def run_mixer_in_cuts(mixer, hs, cuts, dtype, page_tokens=16):
     """Feeds two sequences (``hs``: [steps, width] each) to a mixer part in steps: ``cuts`` lists, per step, how
     many rows of each sequence it brings (0: the sequence sits the step out).  Sequence 0 lives in state slot 2,
     sequence 1 in slot 0; their pages are interleaved.  Returns each sequence's outputs in order."""
     need = mixer.cache_need()
-    made = views_of(need, dtype=dtype)
+    made = views_of(need, page_tokens=page_tokens, dtype=dtype)
     pages = {0: list(range(1, 40, 2)), 1: list(range(0, 40, 2))}
     at, outs = [0, 0], [[], []]
     for cut in cuts:
@@ -274,7 +274,7 @@ def run_mixer_in_cuts(mixer, hs, cuts, dtype):
             rows.append(hs[s][at[s]:at[s] + cut[s]])
         table = torch.tensor([pages[s] for s in present], dtype=torch.int32, device=DEV)
         step = step_of(meta, dtype, [(2, 0)[s] for s in present], {0: table})
-        result = mixer.forward(torch.cat(rows).to(DEV).to(dtype), step, nested(need, made, table))
+        result = mixer.forward(torch.cat(rows).to(DEV).to(dtype), step, nested(need, made, table, page_tokens))
         first = 0
         for s in present:
             outs[s].append(result[first:first + cut[s]].float().cpu())
