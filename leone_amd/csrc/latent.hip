@@ -353,19 +353,28 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
             // ---- S^T = K Q^T for the two 16-key halves ----
             const int ka = 8 * (c >> 2) + (c & 3);                // this lane's key of the first half; the second's is 4 further
             const bf16_t* kp = k_pool + page * key_page + static_cast<long>(tok0 + ka) * 8;
+            // All of a tile's keys are asked for before the first product waits for any (no branch stands between the
+            // loads): steps beyond the latent's width read a step that exists and meet zero queries.
+            lat_bf16x8 xa[kSteps], xb[kSteps];
+#pragma unroll
+            for (int s = 0; s < kSteps; ++s) {
+                const bf16_t* from = kp + static_cast<long>(4 * min(s, steps - 1) + g) * page_tokens * 8;
+                xa[s] = lat_load8(from);
+                xb[s] = lat_load8(from + 32);
+            }
+            if (!inner) {                                         // what lies outside the range may hold anything
+                const bool drop_a = key0 + ka < lo || key0 + ka > hi, drop_b = key0 + ka + 4 < lo || key0 + ka + 4 > hi;
+#pragma unroll
+                for (int s = 0; s < kSteps; ++s) {
+                    if (drop_a) xa[s] = lat_zero8();
+                    if (drop_b) xb[s] = lat_zero8();
+                }
+            }
             lat_floatx4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int s = 0; s < kSteps; ++s) {
-                if (s < steps) {
-                    const bf16_t* from = kp + static_cast<long>(4 * s + g) * page_tokens * 8;
-                    lat_bf16x8 xa = lat_load8(from), xb = lat_load8(from + 32);
-                    if (!inner) {                                 // what lies outside the range may hold anything
-                        if (key0 + ka < lo || key0 + ka > hi) xa = lat_zero8();
-                        if (key0 + ka + 4 < lo || key0 + ka + 4 > hi) xb = lat_zero8();
-                    }
-                    sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa, qreg[s], sa, 0, 0, 0);
-                    sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb, qreg[s], sb, 0, 0, 0);
-                }
+                sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[s], qreg[s], sa, 0, 0, 0);
+                sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb[s], qreg[s], sb, 0, 0, 0);
             }
             // lane (g, c) holds, for column c, the scores of keys key0 + 8g + j, j = 0 .. 7
             const int run0 = key0 + 8 * g;
@@ -403,19 +412,29 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
                     keep[i] = ((e0 >= lo && e0 <= hi) ? 0x0000ffffu : 0u) | ((e1 >= lo && e1 <= hi) ? 0xffff0000u : 0u);
                 }
             }
+            // eight 16-element runs of the values at a time, asked for together; runs beyond the latent read one that exists
+            // into sums that nobody reads
+            constexpr int kBatch = kDT < 8 ? kDT : 8;
 #pragma unroll
-            for (int dt = 0; dt < kDT; ++dt) {
-                if (dt < dts) {
-                    uint4 raw = *reinterpret_cast<const uint4*>(vp + static_cast<long>(16 * dt) * 8);
-                    if (!inner) {
-                        raw.x &= keep[0];
-                        raw.y &= keep[1];
-                        raw.z &= keep[2];
-                        raw.w &= keep[3];
+            for (int dt0 = 0; dt0 < kDT; dt0 += kBatch) {
+                uint4 raw[kBatch];
+#pragma unroll
+                for (int i = 0; i < kBatch; ++i)
+                    raw[i] = *reinterpret_cast<const uint4*>(vp + static_cast<long>(16 * min(dt0 + i, dts - 1)) * 8);
+                if (!inner) {
+#pragma unroll
+                    for (int i = 0; i < kBatch; ++i) {
+                        raw[i].x &= keep[0];
+                        raw[i].y &= keep[1];
+                        raw[i].z &= keep[2];
+                        raw[i].w &= keep[3];
                     }
+                }
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[dt][r] *= alpha;
-                    acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lat_bf16x8, raw), pt, acc[dt], 0, 0, 0);
+                for (int i = 0; i < kBatch; ++i) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[dt0 + i][r] *= alpha;
+                    acc[dt0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lat_bf16x8, raw[i]), pt, acc[dt0 + i], 0, 0, 0);
                 }
             }
         }
