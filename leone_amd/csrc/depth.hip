@@ -17,55 +17,141 @@ namespace leone {
 
 constexpr int kDepthThreads = 256;
 
-template <typename TY>
+// A thread holds up to kHold runs of kRun elements of its row in registers between the two passes (rows of up to
+// 256 * kHold * kRun elements; longer rows read the stream a second time): every read of the first pass is asked for
+// before any is used, so a row is one trip to memory.
+template <typename TY, int kRun>
 __global__ void __launch_bounds__(kDepthThreads)
 residual_norm_kernel(float* __restrict__ x, const float* __restrict__ delta, int planes, long plane, float scale, AnyVec gain,
                      float eps, TY* __restrict__ y, const int* __restrict__ rows, int hidden) {
+    constexpr int kHold = 4;
     __shared__ float scratch[kDepthThreads / kWave];
     const int out_row = blockIdx.x;
     const long in_row = rows ? rows[out_row] : out_row;
     float* xr = x + in_row * hidden;
     const float* dr = delta ? delta + in_row * hidden : nullptr;
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < hidden; c += kDepthThreads) {
-        float v = xr[c];
-        if (dr) {
-            float d = 0.f;
-            for (int p = 0; p < planes; ++p) d += dr[p * plane + c];
-            v = fmaf(scale, d, v);
-            if (!rows) xr[c] = v;
+    auto load = [](const float* p, float* to) {
+        if constexpr (kRun == 4) {
+            const float4 v = *reinterpret_cast<const float4*>(p);
+            to[0] = v.x, to[1] = v.y, to[2] = v.z, to[3] = v.w;
+        } else {
+            to[0] = *p;
         }
-        ss = fmaf(v, v, ss);
+    };
+    auto sum_of = [&](int c, float* v) {           // the stream's elements from c on with the delta added
+        load(xr + c, v);
+        if (dr) {
+            float d[kRun], part[kRun];
+#pragma unroll
+            for (int i = 0; i < kRun; ++i) d[i] = 0.f;
+            for (int p = 0; p < planes; ++p) {
+                load(dr + p * plane + c, part);
+#pragma unroll
+                for (int i = 0; i < kRun; ++i) d[i] += part[i];
+            }
+#pragma unroll
+            for (int i = 0; i < kRun; ++i) v[i] = fmaf(scale, d[i], v[i]);
+        }
+    };
+    const int step = kDepthThreads * kRun;
+    float held[kHold][kRun];
+    float ss = 0.f;
+#pragma unroll
+    for (int h = 0; h < kHold; ++h) {
+        const int c = threadIdx.x * kRun + h * step;
+        if (c < hidden) sum_of(c, held[h]);
+    }
+#pragma unroll
+    for (int h = 0; h < kHold; ++h) {
+        const int c = threadIdx.x * kRun + h * step;
+        if (c < hidden) {
+#pragma unroll
+            for (int i = 0; i < kRun; ++i) {
+                ss = fmaf(held[h][i], held[h][i], ss);
+                if (dr && !rows) xr[c + i] = held[h][i];
+            }
+        }
+    }
+    for (int c = threadIdx.x * kRun + kHold * step; c < hidden; c += step) {
+        float v[kRun];
+        sum_of(c, v);
+#pragma unroll
+        for (int i = 0; i < kRun; ++i) {
+            ss = fmaf(v[i], v[i], ss);
+            if (dr && !rows) xr[c + i] = v[i];
+        }
     }
     if (!y) return;
     const float inv = 1.0f / sqrtf(block_sum<kDepthThreads>(ss, scratch) / static_cast<float>(hidden) + eps);
     TY* yr = y + static_cast<long>(out_row) * hidden;
-    for (int c = threadIdx.x; c < hidden; c += kDepthThreads) {
-        float v = xr[c];
-        if (dr && rows) {
-            float d = 0.f;
-            for (int p = 0; p < planes; ++p) d += dr[p * plane + c];
-            v = fmaf(scale, d, v);
+#pragma unroll
+    for (int h = 0; h < kHold; ++h) {
+        const int c = threadIdx.x * kRun + h * step;
+        if (c < hidden) {
+#pragma unroll
+            for (int i = 0; i < kRun; ++i) yr[c + i] = from_float<TY>(held[h][i] * inv * load_any(gain, c + i));
         }
-        yr[c] = from_float<TY>(v * inv * load_any(gain, c));
+    }
+    for (int c = threadIdx.x * kRun + kHold * step; c < hidden; c += step) {
+        float v[kRun];
+        if (dr && rows) {
+            sum_of(c, v);
+        } else {
+#pragma unroll
+            for (int i = 0; i < kRun; ++i) v[i] = xr[c + i];
+        }
+#pragma unroll
+        for (int i = 0; i < kRun; ++i) yr[c + i] = from_float<TY>(v[i] * inv * load_any(gain, c + i));
     }
 }
 
+// kRun elements a thread (4 where the sizes allow 16-byte accesses, else 1).
+template <int kRun>
 __global__ void __launch_bounds__(kDepthThreads)
 depth_mix_kernel(float* __restrict__ x, const float* __restrict__ delta, int planes, long plane, float scale,
                  float* __restrict__ history, long slot_stride, int count, AnyVec weight, long total) {
-    const long at = static_cast<long>(blockIdx.x) * kDepthThreads + threadIdx.x;
+    const long at = (static_cast<long>(blockIdx.x) * kDepthThreads + threadIdx.x) * kRun;
     if (at >= total) return;
-    float own = x[at];
+    float own[kRun], sum[kRun];
+    auto load = [](const float* p, float* to) {
+        if constexpr (kRun == 4) {
+            const float4 v = *reinterpret_cast<const float4*>(p);
+            to[0] = v.x, to[1] = v.y, to[2] = v.z, to[3] = v.w;
+        } else {
+            to[0] = *p;
+        }
+    };
+    auto store = [](float* p, const float* from) {
+        if constexpr (kRun == 4) *reinterpret_cast<float4*>(p) = float4{from[0], from[1], from[2], from[3]};
+        else *p = from[0];
+    };
+    load(x + at, own);
     if (delta) {
-        float d = 0.f;
-        for (int p = 0; p < planes; ++p) d += delta[p * plane + at];
-        own = fmaf(scale, d, own);
+        float d[kRun], part[kRun];
+#pragma unroll
+        for (int i = 0; i < kRun; ++i) d[i] = 0.f;
+        for (int p = 0; p < planes; ++p) {
+            load(delta + p * plane + at, part);
+#pragma unroll
+            for (int i = 0; i < kRun; ++i) d[i] += part[i];
+        }
+#pragma unroll
+        for (int i = 0; i < kRun; ++i) own[i] = fmaf(scale, d[i], own[i]);
     }
-    history[static_cast<long>(count - 1) * slot_stride + at] = own;
-    float sum = 0.f;
-    for (int j = 0; j + 1 < count; ++j) sum = fmaf(load_any(weight, j), history[j * slot_stride + at], sum);
-    x[at] = fmaf(load_any(weight, count - 1), own, sum);
+    store(history + static_cast<long>(count - 1) * slot_stride + at, own);
+#pragma unroll
+    for (int i = 0; i < kRun; ++i) sum[i] = 0.f;
+    for (int j = 0; j + 1 < count; ++j) {
+        float kept[kRun];
+        load(history + j * slot_stride + at, kept);
+        const float w = load_any(weight, j);
+#pragma unroll
+        for (int i = 0; i < kRun; ++i) sum[i] = fmaf(w, kept[i], sum[i]);
+    }
+    const float last = load_any(weight, count - 1);
+#pragma unroll
+    for (int i = 0; i < kRun; ++i) sum[i] = fmaf(last, own[i], sum[i]);
+    store(x + at, sum);
 }
 
 }  // namespace leone
@@ -80,12 +166,19 @@ extern "C" int leone_residual_norm(float* x, const float* delta, int planes, lon
     LEONE_REQUIRE(!y || (gain && eps > 0.f && (gain_dtype == kF32 || gain_dtype == kBF16) && (y_dtype == kF32 || y_dtype == kBF16)),
                   "residual_norm: a norm needs a gain, eps and known types");
     LEONE_REQUIRE(!rows || y, "residual_norm: picked rows come with a norm");
-    if (y_dtype == kBF16 && y)
-        residual_norm_kernel<bf16_t><<<n_rows, kDepthThreads, 0, stream>>>(x, delta, planes, plane, scale, AnyVec{gain, gain_dtype},
-                                                                         eps, static_cast<bf16_t*>(y), rows, hidden);
-    else
-        residual_norm_kernel<float><<<n_rows, kDepthThreads, 0, stream>>>(x, delta, planes, plane, scale, AnyVec{gain, gain_dtype},
-                                                                        eps, static_cast<float*>(y), rows, hidden);
+    const bool runs = hidden % 4 == 0 && plane % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(delta) % 16 == 0;
+#define LEONE_RESIDUAL_NORM(TY, R)                                                                                      \
+    residual_norm_kernel<TY, R><<<n_rows, kDepthThreads, 0, stream>>>(x, delta, planes, plane, scale, AnyVec{gain, gain_dtype}, \
+                                                                    eps, static_cast<TY*>(y), rows, hidden)
+    if (y_dtype == kBF16 && y) {
+        if (runs) LEONE_RESIDUAL_NORM(bf16_t, 4);
+        else LEONE_RESIDUAL_NORM(bf16_t, 1);
+    } else {
+        if (runs) LEONE_RESIDUAL_NORM(float, 4);
+        else LEONE_RESIDUAL_NORM(float, 1);
+    }
+#undef LEONE_RESIDUAL_NORM
     LEONE_LAUNCH_CHECK("residual_norm");
     return 0;
 }
@@ -96,10 +189,17 @@ extern "C" int leone_depth_mix(float* x, const float* delta, int planes, long pl
     LEONE_REQUIRE(x && history && weight && total > 0 && count >= 1 && slot_stride >= total, "depth_mix: null pointer or empty sizes");
     LEONE_REQUIRE(weight_dtype == kF32 || weight_dtype == kBF16, "depth_mix: unknown type of the weights");
     LEONE_REQUIRE(!delta || (planes >= 1 && planes <= 16), "depth_mix: %d planes of what is to be added", planes);
-    const long blocks = (total + kDepthThreads - 1) / kDepthThreads;
+    const bool runs = total % 4 == 0 && slot_stride % 4 == 0 && plane % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(history) % 16 == 0 && reinterpret_cast<uintptr_t>(delta) % 16 == 0;
+    const long threads = runs ? total / 4 : total;
+    const long blocks = (threads + kDepthThreads - 1) / kDepthThreads;
     LEONE_REQUIRE(blocks <= 0x7fffffffL, "depth_mix: %ld elements are too many", total);
-    depth_mix_kernel<<<static_cast<unsigned>(blocks), kDepthThreads, 0, stream>>>(x, delta, planes, plane, scale, history,
-                                                                                 slot_stride, count, AnyVec{weight, weight_dtype}, total);
+    if (runs)
+        depth_mix_kernel<4><<<static_cast<unsigned>(blocks), kDepthThreads, 0, stream>>>(x, delta, planes, plane, scale, history,
+                                                                                        slot_stride, count, AnyVec{weight, weight_dtype}, total);
+    else
+        depth_mix_kernel<1><<<static_cast<unsigned>(blocks), kDepthThreads, 0, stream>>>(x, delta, planes, plane, scale, history,
+                                                                                        slot_stride, count, AnyVec{weight, weight_dtype}, total);
     LEONE_LAUNCH_CHECK("depth_mix");
     return 0;
 }

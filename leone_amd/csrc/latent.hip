@@ -91,55 +91,126 @@ latent_prepare_kernel(const float* __restrict__ proj, long stride, int q_off, in
 }
 
 constexpr int kHpRows = 8;
-constexpr int kHpCols = 64;          // output columns a workgroup takes; its four waves split the inner elements
+
+// Eight neighbouring weights of one inner element as floats: one 16- or 32-byte read where `runs` says the rows of the
+// matrix allow it, element by element (zeros beyond `valid`) otherwise.
+template <typename TW>
+__device__ inline void load_weights8(const TW* p, int valid, bool runs, float* to) {
+    if (runs && valid >= 8) {
+        if constexpr (sizeof(TW) == 2) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(p);
+            const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                to[2 * i] = __uint_as_float(w[i] << 16);
+                to[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+            }
+        } else {
+            const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+            to[0] = a.x, to[1] = a.y, to[2] = a.z, to[3] = a.w, to[4] = b.x, to[5] = b.y, to[6] = b.z, to[7] = b.w;
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) to[j] = j < valid ? to_float(p[j]) : 0.f;
+}
 
 // x: [rows] rows of x_row_stride floats or TX, head h's `inner` elements at h * x_head_stride; w: [heads][inner][outer]
 // (null: only the tail is handed on); y: rows of y_row_stride, head h's results at h * y_head_stride.  A workgroup takes
-// 8 rows, one head and 64 columns; a lane owns a column, a wave a quarter of the inner elements; the waves' sums are
-// added in their order.
-template <typename TX, typename TW, typename TY>
+// 8 rows, one head and 8 * kGroups columns.  A thread owns 8 neighbouring columns and every (256 / kGroups)th inner
+// element, so that a wave reads whole runs of the matrix and a thread's reads are on their way together: the first
+// four are asked for before the rows are staged (they do not depend on them; a step of few rows is a chain of a few
+// trips to memory and nothing else).  The partial sums of a result are added over a wave's lanes by shuffles and over
+// the waves, in their order, in shared memory.  Deep products (W_uv on the weighted sums) take kGroups = 2, flat ones 8.
+template <typename TX, typename TW, typename TY, int kGroups>
 __global__ void __launch_bounds__(kLatThreads)
 head_product_kernel(const TX* __restrict__ x, long x_row_stride, long x_head_stride, const TW* __restrict__ w,
                     TY* __restrict__ y, long y_row_stride, long y_head_stride, int rows, int inner, int outer, int tail,
                     const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot_half,
-                    int table_positions, const int* __restrict__ positions) {
-    extern __shared__ __align__(16) float hp_lds[];            // [kHpRows][inner + tail], then [waves][kHpRows][kHpCols]
+                    int table_positions, const int* __restrict__ positions, int runs) {
+    constexpr int kCols = 8 * kGroups, kSlices = kLatThreads / kGroups, kAhead = 4;
+    extern __shared__ __align__(16) float hp_lds[];            // [kHpRows][inner + tail], then [waves][kHpRows][kCols]
     const int head = blockIdx.y, row0 = blockIdx.x * kHpRows;
     const int here = min(kHpRows, rows - row0);
     const int width = inner + tail;
     float* partial = hp_lds + kHpRows * width;
-    for (int idx = threadIdx.x; idx < kHpRows * width; idx += kLatThreads) {
-        const int r = idx / width, k = idx % width;
-        hp_lds[idx] = r < here ? to_float(x[(row0 + r) * x_row_stride + head * x_head_stride + k]) : 0.f;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int group = threadIdx.x % kGroups, slice = threadIdx.x / kGroups;
+    const int n0 = blockIdx.z * kCols + group * 8;
+    const int valid = w ? min(8, outer - n0) : 0;
+    const TW* wh = w ? w + static_cast<long>(head) * inner * outer + n0 : nullptr;
+    float ahead[kAhead][8];
+#pragma unroll
+    for (int i = 0; i < kAhead; ++i) {
+        const int k = slice + i * kSlices;
+        if (valid > 0 && k < inner) {
+            load_weights8(wh + static_cast<long>(k) * outer, valid, runs != 0, ahead[i]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ahead[i][j] = 0.f;
+        }
+    }
+    // eight elements a thread are asked for before the first is put away: a read a trip would be a trip to memory each
+    constexpr int kStage = 8;
+    for (int base = threadIdx.x; base < kHpRows * width; base += kLatThreads * kStage) {
+        float staged[kStage];
+#pragma unroll
+        for (int i = 0; i < kStage; ++i) {
+            const int idx = base + i * kLatThreads;
+            const int r = idx / width, k = idx % width;
+            staged[i] = (idx < kHpRows * width && r < here) ? to_float(x[(row0 + r) * x_row_stride + head * x_head_stride + k]) : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < kStage; ++i)
+            if (base + i * kLatThreads < kHpRows * width) hp_lds[base + i * kLatThreads] = staged[i];
     }
     __syncthreads();
     if (w) {
-        const int lane = threadIdx.x % kWave, part = threadIdx.x / kWave;
-        const int n = blockIdx.z * kHpCols + lane;
-        const int share = (inner + kLatWaves - 1) / kLatWaves;
-        const int k0 = part * share, k1 = min(inner, k0 + share);
-        float acc[kHpRows];
+        float acc[kHpRows][8];
 #pragma unroll
-        for (int r = 0; r < kHpRows; ++r) acc[r] = 0.f;
-        if (n < outer) {
-            const TW* wh = w + static_cast<long>(head) * inner * outer + n;
+        for (int r = 0; r < kHpRows; ++r)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[r][j] = 0.f;
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+            const int k = min(slice + i * kSlices, inner - 1);     // beyond the inner size the weights are zeros
+#pragma unroll
+            for (int r = 0; r < kHpRows; ++r) {
+                const float xv = hp_lds[r * width + k];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[r][j] = fmaf(xv, ahead[i][j], acc[r][j]);
+            }
+        }
+        if (valid > 0) {
 #pragma unroll 4
-            for (int k = k0; k < k1; ++k) {
-                const float wv = to_float(wh[static_cast<long>(k) * outer]);
+            for (int k = slice + kAhead * kSlices; k < inner; k += kSlices) {
+                float wv[8];
+                load_weights8(wh + static_cast<long>(k) * outer, valid, runs != 0, wv);
 #pragma unroll
-                for (int r = 0; r < kHpRows; ++r) acc[r] = fmaf(hp_lds[r * width + k], wv, acc[r]);
+                for (int r = 0; r < kHpRows; ++r) {
+                    const float xv = hp_lds[r * width + k];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[r][j] = fmaf(xv, wv[j], acc[r][j]);
+                }
             }
         }
 #pragma unroll
-        for (int r = 0; r < kHpRows; ++r) partial[(part * kHpRows + r) * kHpCols + lane] = acc[r];
+        for (int r = 0; r < kHpRows; ++r)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float v = acc[r][j];
+#pragma unroll
+                for (int off = kGroups; off < kWave; off <<= 1) v += __shfl_xor(v, off, kWave);
+                if (lane < kGroups) partial[(wave * kHpRows + r) * kCols + group * 8 + j] = v;
+            }
         __syncthreads();
-        for (int idx = threadIdx.x; idx < here * kHpCols; idx += kLatThreads) {
-            const int r = idx / kHpCols, col = idx % kHpCols;
-            if (blockIdx.z * kHpCols + col >= outer) continue;
+        for (int idx = threadIdx.x; idx < here * kCols; idx += kLatThreads) {
+            const int r = idx / kCols, col = idx % kCols;
+            if (blockIdx.z * kCols + col >= outer) continue;
             float sum = 0.f;
 #pragma unroll
-            for (int p = 0; p < kLatWaves; ++p) sum += partial[(p * kHpRows + r) * kHpCols + col];
-            y[(row0 + r) * y_row_stride + head * y_head_stride + blockIdx.z * kHpCols + col] = from_float<TY>(sum);
+            for (int p = 0; p < kLatWaves; ++p) sum += partial[(p * kHpRows + r) * kCols + col];
+            y[(row0 + r) * y_row_stride + head * y_head_stride + blockIdx.z * kCols + col] = from_float<TY>(sum);
         }
     }
     if (blockIdx.z != 0) return;
@@ -300,7 +371,8 @@ __global__ void __launch_bounds__(kLatThreads)
 latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ out, const bf16_t* __restrict__ k_pool,
                               const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
                               const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
-                              int total, int heads, int rank, int width, int page_tokens, float to_log2, int window) {
+                              int total, int heads, int rank, int width, int page_tokens, float to_log2, int window,
+                              int splits, float* __restrict__ part_acc, float* __restrict__ part_ml) {
     extern __shared__ __align__(16) float lc_lds[];               // [16][rank + 4] sums, then [waves][16] maxima, [waves][16] sums
     const int pitch = rank + 4;
     float* sm_acc = lc_lds;
@@ -341,7 +413,8 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
             lo = min(lo, __shfl_xor(lo, off, kWave));
         }
         const int* table = block_table + static_cast<long>(walked) * max_blocks;
-        for (int t = lo / kCoreTile + wave; t <= hi / kCoreTile; t += kLatWaves) {
+        // the tiles go round the waves of all the workgroups that share these columns (blockIdx.y: one of `splits`)
+        for (int t = lo / kCoreTile + blockIdx.y * kLatWaves + wave; t <= hi / kCoreTile; t += kLatWaves * splits) {
             const int key0 = t * kCoreTile;
             const int page = table[key0 / page_tokens];
             const int tok0 = key0 % page_tokens;
@@ -376,14 +449,36 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
                 sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[s], qreg[s], sa, 0, 0, 0);
                 sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xb[s], qreg[s], sb, 0, 0, 0);
             }
-            // lane (g, c) holds, for column c, the scores of keys key0 + 8g + j, j = 0 .. 7
+            // The tile's values are asked for now, all of them, into the registers the keys have left: they arrive while
+            // the softmax is worked out.  Runs beyond the latent read one that exists, into sums that nobody reads.
             const int run0 = key0 + 8 * g;
+            const bf16_t* vp = v_pool + page * value_page + (static_cast<long>((tok0 + 8 * g) / 8) * rank + c) * 8;
+            uint4 raw[kDT];
+#pragma unroll
+            for (int dt = 0; dt < kDT; ++dt)
+                raw[dt] = *reinterpret_cast<const uint4*>(vp + static_cast<long>(16 * min(dt, dts - 1)) * 8);
+            if (!inner) {                                         // slots outside the range may hold anything, even NaN
+                unsigned keep[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int e0 = run0 + 2 * i, e1 = e0 + 1;
+                    keep[i] = ((e0 >= lo && e0 <= hi) ? 0x0000ffffu : 0u) | ((e1 >= lo && e1 <= hi) ? 0xffff0000u : 0u);
+                }
+#pragma unroll
+                for (int dt = 0; dt < kDT; ++dt) {
+                    raw[dt].x &= keep[0];
+                    raw[dt].y &= keep[1];
+                    raw[dt].z &= keep[2];
+                    raw[dt].w &= keep[3];
+                }
+            }
+            // lane (g, c) holds, for column c, the scores of keys key0 + 8g + j, j = 0 .. 7
             float sc[8], tile_max = -INFINITY;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int key = run0 + j;
-                const float raw = j < 4 ? sa[j & 3] : sb[j & 3];
-                sc[j] = (mine && key >= first && key <= pos) ? raw * to_log2 : -INFINITY;
+                const float score = j < 4 ? sa[j & 3] : sb[j & 3];
+                sc[j] = (mine && key >= first && key <= pos) ? score * to_log2 : -INFINITY;
                 tile_max = fmaxf(tile_max, sc[j]);
             }
             tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
@@ -403,39 +498,11 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
             l_run = l_run * alpha + psum;
             m_run = m_new;
             // ---- O^T += V^T P^T ----
-            const bf16_t* vp = v_pool + page * value_page + (static_cast<long>((tok0 + 8 * g) / 8) * rank + c) * 8;
-            unsigned keep[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-            if (!inner) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int e0 = run0 + 2 * i, e1 = e0 + 1;
-                    keep[i] = ((e0 >= lo && e0 <= hi) ? 0x0000ffffu : 0u) | ((e1 >= lo && e1 <= hi) ? 0xffff0000u : 0u);
-                }
-            }
-            // eight 16-element runs of the values at a time, asked for together; runs beyond the latent read one that exists
-            // into sums that nobody reads
-            constexpr int kBatch = kDT < 8 ? kDT : 8;
+            for (int dt = 0; dt < kDT; ++dt) {
 #pragma unroll
-            for (int dt0 = 0; dt0 < kDT; dt0 += kBatch) {
-                uint4 raw[kBatch];
-#pragma unroll
-                for (int i = 0; i < kBatch; ++i)
-                    raw[i] = *reinterpret_cast<const uint4*>(vp + static_cast<long>(16 * min(dt0 + i, dts - 1)) * 8);
-                if (!inner) {
-#pragma unroll
-                    for (int i = 0; i < kBatch; ++i) {
-                        raw[i].x &= keep[0];
-                        raw[i].y &= keep[1];
-                        raw[i].z &= keep[2];
-                        raw[i].w &= keep[3];
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < kBatch; ++i) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[dt0 + i][r] *= alpha;
-                    acc[dt0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lat_bf16x8, raw[i]), pt, acc[dt0 + i], 0, 0, 0);
-                }
+                for (int r = 0; r < 4; ++r) acc[dt][r] *= alpha;
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lat_bf16x8, raw[dt]), pt, acc[dt], 0, 0, 0);
             }
         }
     }
@@ -456,7 +523,8 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
         const float mw = sm_m[w * 16 + c];
         denom += sm_l[w * 16 + c] * (mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - top));
     }
-    const float weight = (m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - top)) / denom;
+    // one workgroup a tile of columns: the result itself; several: sums against the workgroup's maximum, for the merge
+    const float weight = (m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - top)) / (splits == 1 ? denom : 1.f);
     for (int w = 0; w < kLatWaves; ++w) {
         if (wave == w) {
 #pragma unroll
@@ -475,24 +543,67 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
         __syncthreads();
     }
     const long pair0 = static_cast<long>(blockIdx.x) * 16;
+    if (splits == 1) {
+        for (int i = threadIdx.x; i < 16 * rank; i += kLatThreads) {
+            const int col = i / rank, e = i % rank;
+            if (pair0 + col < total) out[(pair0 + col) * rank + e] = sm_acc[col * pitch + e];
+        }
+        return;
+    }
+    const long mine_at = (static_cast<long>(blockIdx.x) * splits + blockIdx.y) * 16;
     for (int i = threadIdx.x; i < 16 * rank; i += kLatThreads) {
         const int col = i / rank, e = i % rank;
-        if (pair0 + col < total) out[(pair0 + col) * rank + e] = sm_acc[col * pitch + e];
+        part_acc[(mine_at + col) * rank + e] = sm_acc[col * pitch + e];
+    }
+    if (wave == 0 && g == 0) {
+        part_ml[(mine_at + c) * 2] = top;
+        part_ml[(mine_at + c) * 2 + 1] = denom;
+    }
+}
+
+// The partial results of the workgroups that shared a tile of columns, in their order; one workgroup a column.
+__global__ void __launch_bounds__(kLatThreads)
+latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, float* __restrict__ out, int total,
+                    int rank, int splits) {
+    const int col = blockIdx.y;
+    const long pair = static_cast<long>(blockIdx.x) * 16 + col;
+    if (pair >= total) return;
+    const long first = static_cast<long>(blockIdx.x) * splits * 16 + col;       // + 16 a split
+    float top = -INFINITY;
+    for (int sp = 0; sp < splits; ++sp) top = fmaxf(top, part_ml[(first + 16L * sp) * 2]);
+    float den = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+        const float m = part_ml[(first + 16L * sp) * 2];
+        den += part_ml[(first + 16L * sp) * 2 + 1] * (m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - top));      // NaN: a key without a page
+    }
+    for (int e = threadIdx.x; e < rank; e += kLatThreads) {
+        float num = 0.f;
+        for (int sp = 0; sp < splits; ++sp) {
+            const float m = part_ml[(first + 16L * sp) * 2];
+            num += part_acc[(first + 16L * sp) * rank + e] * (m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - top));
+        }
+        out[pair * rank + e] = num / den;
     }
 }
 
 template <int kSteps, int kDT>
 static int launch_latent_cores(const void* q, float* out, const void* k_pool, const void* v_pool, const int* positions,
                                const int* row_entry, const int* block_table, int max_blocks, int rows, int heads, int rank,
-                               int rot, int page_tokens, float scale, int window, hipStream_t stream) {
+                               int rot, int page_tokens, float scale, int window, int splits, float* part_acc, float* part_ml,
+                               hipStream_t stream) {
     const long total = static_cast<long>(rows) * heads;
     const size_t shared = (static_cast<size_t>(16) * (rank + 4) + 2 * kLatWaves * 16) * sizeof(float);
     LEONE_REQUIRE(shared <= 64 * 1024 && (total + 15) / 16 <= 0x7fffffffL, "latent_attention_cores: %ld pairs, a latent of %d", total, rank);
-    latent_attention_cores_kernel<kSteps, kDT><<<static_cast<unsigned>((total + 15) / 16), kLatThreads, shared, stream>>>(
+    const unsigned tiles = static_cast<unsigned>((total + 15) / 16);
+    latent_attention_cores_kernel<kSteps, kDT><<<dim3(tiles, splits), kLatThreads, shared, stream>>>(
         static_cast<const bf16_t*>(q), out, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), positions,
         row_entry, block_table, max_blocks, static_cast<int>(total), heads, rank, rank + rot, page_tokens,
-        scale * 1.4426950408889634f, window);
+        scale * 1.4426950408889634f, window, splits, part_acc, part_ml);
     LEONE_LAUNCH_CHECK("latent_attention_cores");
+    if (splits > 1) {
+        latent_merge_kernel<<<dim3(tiles, 16), kLatThreads, 0, stream>>>(part_acc, part_ml, out, static_cast<int>(total), rank, splits);
+        LEONE_LAUNCH_CHECK("latent_merge");
+    }
     return 0;
 }
 
@@ -550,14 +661,22 @@ extern "C" int leone_head_product(const float* x, long x_row_stride, long x_head
                   "head_product: rows too short for %d heads of %d + %d in, %d + %d out", heads, inner, tail, outer, tail);
     LEONE_REQUIRE((cos_table == nullptr) == (sin_table == nullptr) && (!cos_table || (rot_half > 0 && 2 * rot_half <= tail && table_positions > 0 && positions)),
                   "head_product: tables for %d pairs of a tail of %d", rot_half, tail);
-    const size_t shared = (static_cast<size_t>(kHpRows) * (inner + tail) + kLatWaves * kHpRows * kHpCols) * sizeof(float);
-    LEONE_REQUIRE(shared <= 64 * 1024 && ceil_div(outer, kHpCols) <= 65535, "head_product: %d + %d elements a head are too many", inner, tail);
-    const dim3 grid(ceil_div(rows, kHpRows), heads, w ? ceil_div(outer, kHpCols) : 1);
+    const int groups = inner >= 256 ? 2 : 8;            // deep products: fewer columns and more of the inner size a workgroup
+    const size_t shared = (static_cast<size_t>(kHpRows) * (inner + tail) + kLatWaves * kHpRows * 8 * groups) * sizeof(float);
+    LEONE_REQUIRE(shared <= 64 * 1024 && ceil_div(outer, 8 * groups) <= 65535, "head_product: %d + %d elements a head are too many", inner, tail);
+    const dim3 grid(ceil_div(rows, kHpRows), heads, w ? ceil_div(outer, 8 * groups) : 1);
     const int half = cos_table ? rot_half : 0;
-#define LEONE_HP(TW, TY)                                                                                               \
-    head_product_kernel<float, TW, TY><<<grid, kLatThreads, shared, stream>>>(                                         \
+    // rows of the matrices that begin on 16-byte borders (32 for float) are read in whole runs
+    const int runs = outer % 8 == 0 && reinterpret_cast<uintptr_t>(w) % 32 == 0;
+#define LEONE_HP_G(TW, TY, G)                                                                                          \
+    head_product_kernel<float, TW, TY, G><<<grid, kLatThreads, shared, stream>>>(                                      \
         x, x_row_stride, x_head_stride, static_cast<const TW*>(w), static_cast<TY*>(y), y_row_stride, y_head_stride, rows, inner, \
-        outer, tail, cos_table, sin_table, half, table_positions, positions)
+        outer, tail, cos_table, sin_table, half, table_positions, positions, runs)
+#define LEONE_HP(TW, TY)                                                                                               \
+    do {                                                                                                               \
+        if (groups == 2) LEONE_HP_G(TW, TY, 2);                                                                        \
+        else LEONE_HP_G(TW, TY, 8);                                                                                    \
+    } while (0)
     if (w_dtype == kF32) {
         if (y_dtype == kF32) LEONE_HP(float, float);
         else LEONE_HP(float, bf16_t);
@@ -566,6 +685,7 @@ extern "C" int leone_head_product(const float* x, long x_row_stride, long x_head
         else LEONE_HP(bf16_t, bf16_t);
     }
 #undef LEONE_HP
+#undef LEONE_HP_G
     LEONE_LAUNCH_CHECK("head_product");
     return 0;
 }
@@ -590,13 +710,17 @@ extern "C" int leone_latent_attention(const float* q, float* out, const void* po
 }
 
 // The same on the matrix cores: bfloat16 queries [rows, heads, rank + rot] and both forms of the cache; rank + rot a
-// multiple of 32 up to leone_latent_cores_max_width(), rank a multiple of 16, pages of a multiple of 32 tokens.
+// multiple of 32 up to leone_latent_cores_max_width(), rank a multiple of 16, pages of a multiple of 32 tokens.  splits
+// > 1: so many workgroups share the keys of every 16 (row, head) pairs; their partial results go through part_acc float32
+// [tiles of 16 pairs, splits, 16, rank] and part_ml [tiles, splits, 16, 2] and a merge.
 extern "C" int leone_latent_cores_max_width() { return 576; }
 
 extern "C" int leone_latent_attention_cores(const void* q, float* out, const void* k_pool, const void* v_pool, const int* positions,
                                             const int* row_entry, const int* block_table, int max_blocks, int rows, int heads,
-                                            int rank, int rot, int page_tokens, float scale, int window, hipStream_t stream) {
+                                            int rank, int rot, int page_tokens, float scale, int window, int splits, float* part_acc,
+                                            float* part_ml, hipStream_t stream) {
     LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table, "latent_attention_cores: null pointer");
+    LEONE_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || (part_acc && part_ml)), "latent_attention_cores: %d workgroups a tile of columns need a workspace", splits);
     LEONE_REQUIRE(rows > 0 && heads > 0 && rank > 0 && rot >= 0 && (rank + rot) % 32 == 0 && rank % 16 == 0 &&
                   rank + rot <= leone_latent_cores_max_width(),
                   "latent_attention_cores: rows %d, %d heads, a latent of %d + %d", rows, heads, rank, rot);
@@ -607,7 +731,7 @@ extern "C" int leone_latent_attention_cores(const void* q, float* out, const voi
     const int width = rank + rot;
 #define LEONE_LATENT_CORES(S, D)                                                                                          \
     return launch_latent_cores<S, D>(q, out, k_pool, v_pool, positions, row_entry, block_table, max_blocks, rows, heads, rank, \
-                                     rot, page_tokens, scale, window, stream)
+                                     rot, page_tokens, scale, window, splits, part_acc, part_ml, stream)
     if (width <= 128) LEONE_LATENT_CORES(4, 8);
     if (width <= 256) LEONE_LATENT_CORES(8, 16);
     LEONE_LATENT_CORES(18, 32);

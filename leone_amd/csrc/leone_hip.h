@@ -331,7 +331,8 @@ int leone_latent_attention(const float* q, float* out, const void* pool, int dty
 int leone_latent_cores_max_width();
 int leone_latent_attention_cores(const void* q, float* out, const void* k_pool, const void* v_pool, const int* positions,
                                  const int* row_entry, const int* block_table, int max_blocks, int rows, int heads, int rank,
-                                 int rot, int page_tokens, float scale, int window, hipStream_t stream);
+                                 int rot, int page_tokens, float scale, int window, int splits, float* part_acc, float* part_ml,
+                                 hipStream_t stream);
 // Residual sums with a factor; the stream as a weighted sum of every earlier layer's result (see depth.hip).
 int leone_residual_norm(float* x, const float* delta, int planes, long plane, float scale, const void* gain, int gain_dtype,
                         float eps, void* y, int y_dtype, const int* rows, int n_rows, int hidden, hipStream_t stream);

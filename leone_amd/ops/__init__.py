@@ -1730,7 +1730,7 @@ def head_product(x: torch.Tensor, weight: torch.Tensor, heads: int, out_dtype: t
     ``[rows, heads * (outer + tail)]`` in ``out_dtype`` with y[r, h, :outer] = x[r, h, :inner] weight[h].  The ``tail``
     elements behind a head's inner ones are handed on behind its outer ones, rotated in neighbouring pairs by the
     row's position if tables come.  Many rows of a bfloat16 model go through the library's batched product (the rows
-    as two bfloat16 parts, float accumulation); the kernel then hands on the tails alone."""
+    rounded to bfloat16, float accumulation); the kernel then hands on the tails alone."""
     rows = x.shape[0]
     if weight.dim() != 3 or weight.shape[0] != heads or x.dim() != 2 or x.shape[1] != heads * (weight.shape[1] + tail):
         raise KernelError(f"head_product: rows {tuple(x.shape)} against {tuple(weight.shape)} for {heads} heads with a tail of {tail}")
@@ -1740,13 +1740,11 @@ def head_product(x: torch.Tensor, weight: torch.Tensor, heads: int, out_dtype: t
     library = weight.dtype == torch.bfloat16 and rows >= HEAD_PRODUCT_LIBRARY_ROWS and inner % 8 == 0 and outer % 8 == 0
     if library:
         with profile.span(profile.LIBRARY_PRODUCT, weight):
-            # the float32 rows as a sum of two bfloat16 parts, so that the result is that of the kernel for few rows
-            # (float32 rows against bfloat16 matrices) up to the order of the sums
             part = x.view(rows, heads, inner + tail)[:, :, :inner]
-            high = part.to(torch.bfloat16)
-            low = (part - high).to(torch.bfloat16)
-            y = torch.bmm(high.transpose(0, 1), weight, out_dtype=torch.float32)
-            y += torch.bmm(low.transpose(0, 1), weight, out_dtype=torch.float32)
+            if part.dtype != torch.bfloat16:
+                part = part.to(torch.bfloat16)
+            y = torch.bmm(part.transpose(0, 1), weight) if out_dtype == torch.bfloat16 else \
+                torch.bmm(part.transpose(0, 1), weight, out_dtype=torch.float32)
             out.view(rows, heads, outer + tail)[:, :, :outer].copy_(y.transpose(0, 1))
         if not tail:
             return out
@@ -1764,14 +1762,29 @@ def latent_cores_supported(dtype: torch.dtype, rank: int, rot: int, page_tokens:
             and rank + rot <= library().leone_latent_cores_max_width())
 
 
+LATENT_SPLIT_TILES = 1       # a wave of the matrix-core kernel keeps at least this many 32-key tiles when keys are shared out
+LATENT_MAX_SPLITS = 16
+
+
+def latent_splits(pairs: int, keys: int, units: int = 256) -> int:
+    """How many workgroups share the keys of every 16 (row, head) pairs: one where the tiles of pairs fill the GPU by
+    themselves, more in steps of few rows over long contexts."""
+    tiles = -(-pairs // 16)
+    by_room = units // max(tiles, 1)
+    by_work = -(-keys // 32) // (4 * LATENT_SPLIT_TILES)
+    return max(1, min(by_room, by_work, LATENT_MAX_SPLITS))
+
+
 def latent_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
                      row_entry: torch.Tensor, block_table: torch.Tensor, heads: int, rank: int, rot: int, scale: float,
-                     window: int = 0) -> torch.Tensor:
+                     window: int = 0, max_position: Optional[int] = None) -> torch.Tensor:
     """Softmax attention over a cache of latents shared by the heads: ``q`` ``[rows, heads * (rank + rot)]`` (the keys'
     up-projection already on the query's side, see ``head_product``), the cache in its two forms (``latent_prepare``);
     a row sees the latents of its request at positions pos - window < j <= pos (``window`` 0: all).  Returns float32
     ``[rows, heads * rank]``: every head's weighted sum of the latents.  bfloat16 queries go to the matrix-core kernel
-    (``latent_cores_supported``), float32 queries to the kernel for any size and type of cache."""
+    (``latent_cores_supported``), float32 queries to the kernel for any size and type of cache.  ``max_position``: the
+    largest position in the step or a bound on it, known on the host: few rows over many keys are shared out over
+    several workgroups by it (``latent_splits``)."""
     rows = q.shape[0]
     page_tokens = _latent_pools("latent_attention", k_pool, v_pool, rank, rot, None)
     if q.shape[1] != heads * (rank + rot):
@@ -1781,10 +1794,18 @@ def latent_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
         if not latent_cores_supported(k_pool.dtype, rank, rot, page_tokens):
             raise KernelError(f"latent_attention: bfloat16 queries are for the matrix-core kernel, which does not take a "
                               f"{k_pool.dtype} cache of {rank} + {rot} in pages of {page_tokens}")
+        keys = 0 if max_position is None else (min(int(window), max_position + 1) if window else max_position + 1)
+        splits = latent_splits(rows * heads, keys, compute_units(q.device))
+        part_acc = part_ml = None
+        if splits > 1:
+            tiles = -(-rows * heads // 16)
+            part_acc = torch.empty((tiles, splits, 16, rank), dtype=torch.float32, device=q.device)
+            part_ml = torch.empty((tiles, splits, 16, 2), dtype=torch.float32, device=q.device)
         call("leone_latent_attention_cores", _dev(q, "latent queries", torch.bfloat16), _dev(out, "latent sums"),
              _dev(k_pool, "latent keys"), _dev(v_pool, "latent values"), _dev(positions, "positions", torch.int32, (rows,)),
              _dev(row_entry, "row map", torch.int32, (rows,)), _dev(block_table, "block table", torch.int32),
-             block_table.shape[1], rows, heads, int(rank), int(rot), page_tokens, float(scale), int(window), _stream())
+             block_table.shape[1], rows, heads, int(rank), int(rot), page_tokens, float(scale), int(window), splits,
+             _dev(part_acc, "partial sums"), _dev(part_ml, "partial maxima"), _stream())
         return out
     if rank + rot > library().leone_latent_max_width():
         raise KernelError(f"latent_attention: a latent of {rank} + {rot} elements, the kernel takes {library().leone_latent_max_width()}")

@@ -88,7 +88,7 @@ _PROTOTYPES = {
     "leone_gated_chain": [P, c_int, P, ctypes.c_long, P, P, ctypes.c_long, c_int, c_int, c_int, c_int, P],
     "leone_latent_prepare": [P, ctypes.c_long, c_int, c_int, c_int, P, P, c_int, c_int, c_int, P, c_int, c_float, P, P, c_int, c_int,
                              P, P, P, c_int, c_int, P, P, c_int, P],
-    "leone_latent_attention_cores": [P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
+    "leone_latent_attention_cores": [P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, P, P, P],
     "leone_head_product": [P, ctypes.c_long, ctypes.c_long, P, c_int, P, c_int, ctypes.c_long, ctypes.c_long, c_int, c_int, c_int,
                            c_int, c_int, P, P, c_int, c_int, P, P],
     "leone_latent_attention": [P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],

@@ -150,6 +150,7 @@ class LatentAttention(Part):
         q = ops.head_product(q, self.w_uk, self.heads, step.dtype if cores else torch.float32, tail=self.rot_dim,
                              cos=rotation.cos, sin=rotation.sin, positions=step.positions)
         mixed = ops.latent_attention(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry, cache.block_table,
-                                     self.heads, self.kv_rank, self.rot_dim, self.scale, int(self.window or 0))
+                                     self.heads, self.kv_rank, self.rot_dim, self.scale, int(self.window or 0),
+                                     max_position=step.max_position)
         values = ops.head_product(mixed, self.w_uv, self.heads, step.dtype)
         return ops.linear(values, self.w_o, out_dtype=torch.float32)

@@ -334,11 +334,14 @@ def test_latent_attention_alone_in_cuts_of_every_size(m, dtype_name, page_tokens
 @pytest.mark.parametrize("page_tokens", [16, 32])
 @pytest.mark.parametrize("window", [None, 40, 64])
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
-def test_latent_attention_finds_planted_keys(dtype_name, window, page_tokens):
+def test_latent_attention_finds_planted_keys(dtype_name, window, page_tokens, monkeypatch):
     """Keys that answer one query each are planted far back, on both sides of page borders (pages of 16), and at the
     last position a window still holds; a decoy stands one position outside the window of a query, with a value of its
     own, and must not be seen.  Queries come in a prompt's portion and as single decoded tokens.  The plain part of the
     query meets the latent through W_uk; the weights here make that the identity on the first elements."""
+    from leone_amd import ops
+    monkeypatch.setattr(ops, "LATENT_SPLIT_TILES", 1)    # single rows far into a sequence: two workgroups share their keys
+    assert ops.latent_splits(2, 290) == 2 and ops.latent_splits(2, 40) == 1 and ops.latent_splits(16 * 300, 290) == 1
     dtype = DTYPES[dtype_name]
     width, heads, dim, rot, vdim, qr, kr = 48, 2, 12, 32, 16, 24, 32      # a latent of 32 + 32: with pages of 32 the matrix cores
     m = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "q_rank": qr, "kv_rank": kr, "scale": 1.0,
