@@ -381,7 +381,10 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const int c = lane % 16, g = lane / 16;
     const int steps = width / 32, dts = rank / 16;
-    const long pair = static_cast<long>(blockIdx.x) * 16 + c;     // this lane's column: (row, head) pair of the step
+    // (Numbering the workgroups so that each of the chip's dies gets a run of neighbouring tiles was measured: a prompt's
+    // attention took a sixth longer, 2.0 against 1.7 ms for six layers of 2,048 rows.)
+    const int tile = blockIdx.x;
+    const long pair = static_cast<long>(tile) * 16 + c;           // this lane's column: (row, head) pair of the step
     const bool valid = pair < total;
     const int row = valid ? static_cast<int>(pair / heads) : 0;
     const int pos = valid ? positions[row] : -1;
@@ -542,7 +545,7 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
         }
         __syncthreads();
     }
-    const long pair0 = static_cast<long>(blockIdx.x) * 16;
+    const long pair0 = static_cast<long>(tile) * 16;
     if (splits == 1) {
         for (int i = threadIdx.x; i < 16 * rank; i += kLatThreads) {
             const int col = i / rank, e = i % rank;
@@ -550,7 +553,7 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
         }
         return;
     }
-    const long mine_at = (static_cast<long>(blockIdx.x) * splits + blockIdx.y) * 16;
+    const long mine_at = (static_cast<long>(tile) * splits + blockIdx.y) * 16;
     for (int i = threadIdx.x; i < 16 * rank; i += kLatThreads) {
         const int col = i / rank, e = i % rank;
         part_acc[(mine_at + col) * rank + e] = sm_acc[col * pitch + e];

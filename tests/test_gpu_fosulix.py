@@ -517,7 +517,7 @@ def test_scaled_residual_norm_and_stream_mixed_over_depth():
     of the kept results of all layers so far."""
     from leone_amd import ops
     gen = torch.Generator().manual_seed(5)
-    for hidden in (40, 192, 1000):
+    for hidden in (37, 40, 192, 1000, 5000):       # single elements and runs of four; rows longer than a thread holds
         rows, eps = 9, 1e-5
         x = torch.randn(rows, hidden, generator=gen)
         planes = torch.randn(3, rows, hidden, generator=gen)
