@@ -194,15 +194,25 @@ head_product_kernel(const TX* __restrict__ x, long x_row_stride, long x_head_str
                 }
             }
         }
+        // one step of the sum over lanes for all 64 sums before the next: the exchanges of a step do not wait for each other
 #pragma unroll
-        for (int r = 0; r < kHpRows; ++r)
+        for (int off = kGroups; off < kWave; off <<= 1) {
+            float other[kHpRows][8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                float v = acc[r][j];
+            for (int r = 0; r < kHpRows; ++r)
 #pragma unroll
-                for (int off = kGroups; off < kWave; off <<= 1) v += __shfl_xor(v, off, kWave);
-                if (lane < kGroups) partial[(wave * kHpRows + r) * kCols + group * 8 + j] = v;
-            }
+                for (int j = 0; j < 8; ++j) other[r][j] = __shfl_xor(acc[r][j], off, kWave);
+#pragma unroll
+            for (int r = 0; r < kHpRows; ++r)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[r][j] += other[r][j];
+        }
+        if (lane < kGroups) {
+#pragma unroll
+            for (int r = 0; r < kHpRows; ++r)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) partial[(wave * kHpRows + r) * kCols + group * 8 + j] = acc[r][j];
+        }
         __syncthreads();
         for (int idx = threadIdx.x; idx < here * kCols; idx += kLatThreads) {
             const int r = idx / kCols, col = idx % kCols;

@@ -183,6 +183,8 @@ class DecoderModel:
                 family = getattr(part, "family", "layer")
                 resident[family] = resident.get(family, 0) + sum(nbytes(s) for s in part.tensor_specs())
         resident["norm"] = resident.get("norm", 0) + sum(nbytes(s) for s in self.final_norm.tensor_specs())
+        if self.spec.depth_weights is not None:
+            resident["depth"] = sum(nbytes(TensorSpec(name, (at + 2,), VECTOR)) for at, name in enumerate(self.spec.depth_weights))
         decode = dict(resident)
         decode["embed"] = resident["embed"] // self.spec.vocab_size * rows
         if "positions" in decode:

@@ -59,13 +59,13 @@ SMALL = {
         layer(latent(4, 8, 8, 12, 20, 24, base=10000.0, scaling=(8.0, 64, 32.0, 1.0), mask=33, kv_from=0), None),
         layer(latent(2, 16, 4, 8, 12, 40, base=500.0), moe(8, 3, 12, groups=(4, 3), scale=0.7, limit=3.0)),
         layer(latent(3, 16, 4, 24, 30, 40, base=500.0, mask=7, kv_from=3), moe(5, 5, 8)),
-    ], mult=0.3, embed_scale=4.0, taps=4),
+    ], mult=0.35, embed_scale=4.0, taps=4),
     "B": config(96, 130, [
         layer(memory(1, 40, 48), moe(9, 4, 8, groups=(9, 5), scale=2.0)),
         layer(latent(1, 24, 16, 40, 48, 16, base=77.0, scaling=(4.0, 32, 8.0, 2.0), mask=16, dims=8), moe(4, 2, 40, groups=(2, 1))),
         layer(memory(5, 8, 8), None),
         layer(latent(3, 8, 16, 8, 16, 16, base=77.0, scaling=(4.0, 32, 8.0, 2.0), mask=40, kv_from=1, dims=8), moe(6, 2, 20, groups=(1, 1))),
-        layer(latent(2, 32, 32, 32, 24, 64, base=20000.0, scaling=(16.0, 128, 32.0, 1.0)), moe(7, 3, 16, limit=0.5)),
+        layer(latent(2, 32, 32, 32, 24, 64, base=30000.0, scaling=(16.0, 128, 32.0, 1.0)), moe(7, 3, 16, limit=0.5)),
     ], eps=1e-6, mult=1.0, embed_scale=1.0, taps=2),
     "C": config(128, 257, [
         layer(latent(8, 16, 16, 16, 64, 32, base=1000.0, mask=24), moe(16, 4, 32, groups=(8, 3), scale=2.5)),
@@ -79,8 +79,8 @@ SMALL = {
     # experts, so that no rounded router input changes a choice at an early position and, through attention and memory,
     # every later position with it: what differs from the plain results in bfloat16 is then attention's rounding.
     "D": config(128, 300, [
-        layer(latent(4, 16, 32, 16, 32, 96, base=1000.0, scaling=(8.0, 64, 32.0, 1.0), mask=40), moe(4, 4, 32, groups=(2, 2), scale=1.5)),
-        layer(latent(16, 8, 32, 8, 64, 96, base=1000.0, scaling=(8.0, 64, 32.0, 1.0), mask=70, kv_from=0), None),
+        layer(latent(4, 16, 64, 16, 32, 64, base=1000.0, scaling=(8.0, 64, 32.0, 1.0), mask=40), moe(4, 4, 32, groups=(2, 2), scale=1.5)),
+        layer(latent(16, 8, 64, 8, 64, 64, base=1000.0, scaling=(8.0, 64, 32.0, 1.0), mask=70, kv_from=0), None),
         layer(memory(2, 32, 32), moe(3, 3, 32)),
         layer(latent(3, 32, 32, 24, 48, 224, base=500.0), moe(2, 2, 48, limit=1.0)),
         layer(latent(2, 16, 64, 16, 32, 512, base=10000.0, mask=33), None),

@@ -94,7 +94,7 @@ def test_errors_name_the_key(change, field):
 
 def test_stretched_frequencies_against_the_plain_ones():
     from leone_amd.parts import POSITIONS, PartSpec
-    cases = [(32, 20000.0, 8.0, 1024, 32.0, 1.0), (8, 77.0, 4.0, 32, 8.0, 2.0), (64, 1e6, 40.0, 4096, 1.0, 1.0),
+    cases = [(32, 50000.0, 4.0, 2048, 16.0, 2.0), (8, 77.0, 4.0, 32, 8.0, 2.0), (64, 1e6, 40.0, 4096, 1.0, 1.0),
              (4, 10.0, 2.0, 16, 4.0, 1.0), (16, 500.0, 1.0, 64, 32.0, 1.0)]
     for dims, base, factor, original, fast, slow in cases:
         scaling = {"factor": factor, "original": original, "fast": fast, "slow": slow}
@@ -108,8 +108,8 @@ def test_stretched_frequencies_against_the_plain_ones():
         assert torch.allclose(cos.double(), torch.cos(angle) * grow, atol=1e-6)
         assert torch.allclose(sin.double(), torch.sin(angle) * grow, atol=1e-6)
     # the first pairs keep their frequency, the last are slowed by the whole factor
-    freq, _ = plain.rotary_frequencies(32, 20000.0, {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0})
-    assert freq[0] == 1.0 and freq[-1] == pytest.approx(20000.0 ** (-30 / 32) / 8.0)
+    freq, _ = plain.rotary_frequencies(32, 50000.0, {"factor": 4.0, "original": 2048, "fast": 16.0, "slow": 1.0})
+    assert freq[0] == 1.0 and freq[-1] == pytest.approx(50000.0 ** (-30 / 32) / 4.0)
 
 
 def test_plain_pieces_agree_with_one_another():

@@ -441,7 +441,7 @@ def test_gated_memory_alone_in_cuts_of_every_size(m, dtype_name):
         assert err.max() <= (2e-5 if dtype_name == "float32" else 3e-2), (s, int(err.argmax()), float(err.max()))
 
 
-ROUTERS = [{"experts": 8, "top": 2, "scale": 1.5, "groups": {"count": 4, "keep": 3}},
+ROUTERS = [{"experts": 10, "top": 3, "scale": 1.25, "groups": {"count": 5, "keep": 3}},
            {"experts": 5, "top": 1, "scale": 1.0},
            {"experts": 9, "top": 4, "scale": 0.5, "groups": {"count": 9, "keep": 5}},
            {"experts": 72, "top": 6, "scale": 2.5, "groups": {"count": 8, "keep": 3}},
