@@ -540,16 +540,21 @@ latent_attention_cores_kernel(const bf16_t* __restrict__ q, float* __restrict__ 
     const float weight = (m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - top)) / (splits == 1 ? denom : 1.f);
     for (int w = 0; w < kLatWaves; ++w) {
         if (wave == w) {
+            // what the waves before left is read in one go, then added to and written in one go
+            float4 sum[kDT];
+#pragma unroll
+            for (int dt = 0; dt < kDT; ++dt) {
+                const float4* from = reinterpret_cast<const float4*>(sm_acc + c * pitch + 16 * min(dt, dts - 1) + 4 * g);
+                sum[dt] = w == 0 ? float4{0.f, 0.f, 0.f, 0.f} : *from;
+            }
 #pragma unroll
             for (int dt = 0; dt < kDT; ++dt) {
                 if (dt < dts) {
-                    float4* to = reinterpret_cast<float4*>(sm_acc + c * pitch + 16 * dt + 4 * g);
-                    float4 sum = w == 0 ? float4{0.f, 0.f, 0.f, 0.f} : *to;
-                    sum.x += acc[dt][0] * weight;
-                    sum.y += acc[dt][1] * weight;
-                    sum.z += acc[dt][2] * weight;
-                    sum.w += acc[dt][3] * weight;
-                    *to = sum;
+                    sum[dt].x += acc[dt][0] * weight;
+                    sum[dt].y += acc[dt][1] * weight;
+                    sum[dt].z += acc[dt][2] * weight;
+                    sum[dt].w += acc[dt][3] * weight;
+                    *reinterpret_cast<float4*>(sm_acc + c * pitch + 16 * dt + 4 * g) = sum[dt];
                 }
             }
         }
@@ -582,19 +587,31 @@ latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict_
     const long pair = static_cast<long>(blockIdx.x) * 16 + col;
     if (pair >= total) return;
     const long first = static_cast<long>(blockIdx.x) * splits * 16 + col;       // + 16 a split
+    // every split's figures are asked for at once (a loop of as many turns as there are splits would wait for each)
+    constexpr int kMost = 16;
+    float m[kMost], f[kMost], l[kMost];
+#pragma unroll
+    for (int sp = 0; sp < kMost; ++sp) {
+        const bool there = sp < splits;
+        m[sp] = there ? part_ml[(first + 16L * sp) * 2] : -INFINITY;
+        l[sp] = there ? part_ml[(first + 16L * sp) * 2 + 1] : 0.f;
+    }
     float top = -INFINITY;
-    for (int sp = 0; sp < splits; ++sp) top = fmaxf(top, part_ml[(first + 16L * sp) * 2]);
+#pragma unroll
+    for (int sp = 0; sp < kMost; ++sp) top = fmaxf(top, m[sp]);
     float den = 0.f;
-    for (int sp = 0; sp < splits; ++sp) {
-        const float m = part_ml[(first + 16L * sp) * 2];
-        den += part_ml[(first + 16L * sp) * 2 + 1] * (m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - top));      // NaN: a key without a page
+#pragma unroll
+    for (int sp = 0; sp < kMost; ++sp) {
+        f[sp] = m[sp] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[sp] - top);
+        if (sp < splits) den += l[sp] * f[sp];            // NaN: a key in reach had no page
     }
     for (int e = threadIdx.x; e < rank; e += kLatThreads) {
+        float part[kMost];
+#pragma unroll
+        for (int sp = 0; sp < kMost; ++sp) part[sp] = sp < splits ? part_acc[(first + 16L * sp) * rank + e] : 0.f;
         float num = 0.f;
-        for (int sp = 0; sp < splits; ++sp) {
-            const float m = part_ml[(first + 16L * sp) * 2];
-            num += part_acc[(first + 16L * sp) * rank + e] * (m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - top));
-        }
+#pragma unroll
+        for (int sp = 0; sp < kMost; ++sp) num += part[sp] * f[sp];
         out[pair * rank + e] = num / den;
     }
 }
@@ -733,7 +750,7 @@ extern "C" int leone_latent_attention_cores(const void* q, float* out, const voi
                                             int rank, int rot, int page_tokens, float scale, int window, int splits, float* part_acc,
                                             float* part_ml, hipStream_t stream) {
     LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table, "latent_attention_cores: null pointer");
-    LEONE_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || (part_acc && part_ml)), "latent_attention_cores: %d workgroups a tile of columns need a workspace", splits);
+    LEONE_REQUIRE(splits >= 1 && splits <= 16 && (splits == 1 || (part_acc && part_ml)), "latent_attention_cores: %d workgroups a tile of columns need a workspace", splits);
     LEONE_REQUIRE(rows > 0 && heads > 0 && rank > 0 && rot >= 0 && (rank + rot) % 32 == 0 && rank % 16 == 0 &&
                   rank + rot <= leone_latent_cores_max_width(),
                   "latent_attention_cores: rows %d, %d heads, a latent of %d + %d", rows, heads, rank, rot);
