@@ -1771,7 +1771,7 @@ def latent_splits(pairs: int, keys: int, units: int = 256) -> int:
     themselves, more in steps of few rows over long contexts."""
     tiles = -(-pairs // 16)
     by_room = units // max(tiles, 1)
-    by_work = -(-keys // 32) // (4 * LATENT_SPLIT_TILES)
+    by_work = -(-(-(-keys // 32) + 1) // (4 * LATENT_SPLIT_TILES))       # a range of keys seldom begins with a tile: one more
     return max(1, min(by_room, by_work, LATENT_MAX_SPLITS))
 
 

@@ -137,6 +137,37 @@ def test_long_portions_of_the_memory_walked_in_chunks(cases, monkeypatch, name, 
     compare(steps, run_steps(engine, steps), expected, "float32", f"{name} chunked walk {schedule}")
 
 
+ODD = fu.config(100, 301, [
+    fu.layer(fu.latent(3, 10, 6, 10, 37, 45, base=300.0, scaling=(3.0, 50, 7.0, 1.5), mask=13), fu.moe(5, 2, 50, limit=1.3, scale=0.8)),
+    fu.layer(fu.memory(2, 24, 40), None),
+    fu.layer(fu.latent(5, 6, 6, 14, 21, 45, base=300.0, scaling=(3.0, 50, 7.0, 1.5), mask=64, kv_from=0), fu.moe(12, 3, 18, groups=(6, 2), scale=3.0)),
+    fu.layer(fu.latent(1, 20, 2, 4, 9, 7, base=50.0), fu.moe(3, 3, 7)),
+], mult=1.7, embed_scale=0.5, taps=3)
+
+
+@pytest.mark.parametrize("dtype_name", list(DTYPES))
+def test_sizes_that_are_multiples_of_nothing(dtype_name):
+    """Width 100, vocabulary 301, latents of 37, 45, 9 and 7 elements, rotated parts of 6 and 2, experts of 50, 18 and 7,
+    a prompt of 300 tokens (the memory's long portions in chunks), pages of 64 tokens: every kernel's path for sizes
+    that fill no run of 8 or 16."""
+    weights = fu.make_weights(ODD, 3, DTYPES[dtype_name], sharpen=1.5 if dtype_name == "float32" else 1.0)
+    gen = np.random.default_rng(1)
+    requests = {f"r{i}": gen.integers(0, ODD["vocab"], size=n).tolist() for i, n in enumerate([300, 70, 5, 129])}
+    expected = {rid: plain.forward(ODD, widened(weights), toks).numpy() for rid, toks in requests.items()}
+    with tempfile.TemporaryDirectory() as folder:
+        fu.write_dir(folder, ODD, weights)
+        for name in ("whole", "mixed"):
+            steps = SCHEDULES[name](requests)
+            engine = make_engine(folder, dtype_name, max_tokens=schedules.max_live_tokens(steps, 64), page_tokens=64, poison_freed=True)
+            got = schedules.collect(steps, run_steps(engine, steps))
+            errors = np.concatenate([fu.relative_error(np.stack(got[rid]), expected[rid]) for rid in got])
+            assert np.isfinite(errors).all()
+            if dtype_name == "float32":
+                assert errors.max() <= TOLERANCE["float32"], (name, float(errors.max()))
+            else:       # a changed choice of experts moves single positions by far more: the median says what rounding does
+                assert np.median(errors) <= TOLERANCE["bfloat16"], (name, float(np.median(errors)))
+
+
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 def test_pages_and_slots_that_held_another_request(cases, dtype_name):
     """One slot and pages enough for one request: every request runs where the one before it ran, and what freed
@@ -340,8 +371,8 @@ def test_latent_attention_finds_planted_keys(dtype_name, window, page_tokens, mo
     own, and must not be seen.  Queries come in a prompt's portion and as single decoded tokens.  The plain part of the
     query meets the latent through W_uk; the weights here make that the identity on the first elements."""
     from leone_amd import ops
-    monkeypatch.setattr(ops, "LATENT_SPLIT_TILES", 1)    # single rows far into a sequence: two workgroups share their keys
-    assert ops.latent_splits(2, 290) == 2 and ops.latent_splits(2, 40) == 1 and ops.latent_splits(16 * 300, 290) == 1
+    monkeypatch.setattr(ops, "LATENT_SPLIT_TILES", 1)    # single rows far into a sequence: three workgroups share their keys
+    assert ops.latent_splits(2, 290) == 3 and ops.latent_splits(2, 40) == 1 and ops.latent_splits(16 * 300, 290) == 1
     dtype = DTYPES[dtype_name]
     width, heads, dim, rot, vdim, qr, kr = 48, 2, 12, 32, 16, 24, 32      # a latent of 32 + 32: with pages of 32 the matrix cores
     m = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "q_rank": qr, "kv_rank": kr, "scale": 1.0,
