@@ -1,3 +1,3 @@
-from . import fosulix, pamevik, qwen3, zukinex  # noqa: F401  (registers the architecture)
+from . import fosulix, nogidra, pamevik, qwen3, zukinex  # noqa: F401  (registers the architecture)
 from .registry import (Architecture, config_from_dict, config_from_dir, known_architectures, lookup,
                        model_spec_for, register_architecture, unregister_architecture)

@@ -3,3 +3,4 @@ from .qwen3 import Qwen3Config
 from .pamevik import PamevikConfig
 from .zukinex import ZukinexConfig
 from .fosulix import FosulixConfig
+from .nogidra import NogidraConfig

@@ -33,7 +33,8 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
                                       const int* __restrict__ positions, const int* __restrict__ row_entry,
                                       const int* __restrict__ block_table, int max_blocks, int q_heads,
                                       int kv_heads, int head_dim, int v_dim, int page_tokens, float scale, int window,
-                                      const float* __restrict__ gate, long gate_stride, int keep_first, int gate_each) {
+                                      const float* __restrict__ gate, long gate_stride, int keep_first, int gate_each,
+                                      const float* __restrict__ slopes, float temp_coef, int temp_every) {
     __shared__ float sm_m[kRowWaves];
     __shared__ float sm_l[kRowWaves];
     __shared__ float sm_acc[kRowWaves][kRowMaxHeadDim];
@@ -46,6 +47,10 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
     const int pos = positions[row];
     const int* table = block_table + static_cast<long>(row_entry[row]) * max_blocks;
     const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    // a query that grows with its position: the factor 1 + coef * ln(floor((pos + 1) / every) + 1) rides on the scale
+    if (temp_every > 0) scale *= 1.0f + temp_coef * logf(static_cast<float>((pos + 1) / temp_every + 1));
+    // a head's scores are lowered by slope * distance
+    const float slope = slopes ? slopes[head] : 0.f;
 
     const T* qr = q + (static_cast<long>(row) * q_heads + head) * head_dim;
     float qv[kRowDimsPerLane];
@@ -80,7 +85,7 @@ __global__ void attention_rows_kernel(const T* __restrict__ q, T* __restrict__ o
             if (d < head_dim) partial = fmaf(qv[i], to_float(kr[key_offset(token, d, page_tokens)]), partial);
             vv[i] = d < v_dim ? to_float(vr[value_offset(token, d, v_dim)]) : 0.f;
         }
-        const float s = wave_sum(partial) * scale;
+        const float s = wave_sum(partial) * scale - slope * static_cast<float>(pos - j);
         const float m_new = fmaxf(m, s);
         const float alpha = expf(m - m_new);
         const float beta = expf(s - m_new);
@@ -139,6 +144,20 @@ extern "C" int leone_attention_rows_kept(const void* q, void* out, const void* k
                                          int max_blocks, int rows, int q_heads, int kv_heads, int head_dim, int v_dim,
                                          int page_tokens, float scale, int window, const float* gate, long gate_stride,
                                          int keep_first, int gate_each, hipStream_t stream) {
+    return leone_attention_rows_biased(q, out, k_pool, v_pool, dtype, positions, row_entry, block_table, max_blocks, rows,
+                                       q_heads, kv_heads, head_dim, v_dim, page_tokens, scale, window, gate, gate_stride,
+                                       keep_first, gate_each, nullptr, 0.f, 0, stream);
+}
+
+// slopes (float [q_heads], may be null): head h's score for the key at distance d = pos - j is lowered by slopes[h] * d.
+// temp_every > 0: the row's queries count times 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1).
+extern "C" int leone_attention_rows_biased(const void* q, void* out, const void* k_pool, const void* v_pool, int dtype,
+                                           const int* positions, const int* row_entry, const int* block_table,
+                                           int max_blocks, int rows, int q_heads, int kv_heads, int head_dim, int v_dim,
+                                           int page_tokens, float scale, int window, const float* gate, long gate_stride,
+                                           int keep_first, int gate_each, const float* slopes, float temp_coef,
+                                           int temp_every, hipStream_t stream) {
+    LEONE_REQUIRE(temp_every >= 0, "attention_rows: the query factor's period %d must not be negative", temp_every);
     LEONE_REQUIRE(dtype == kF32 || dtype == kBF16, "attention_rows: unknown element type %d", dtype);
     LEONE_REQUIRE(q && out && k_pool && v_pool && positions && row_entry && block_table, "attention_rows: null pointer");
     LEONE_REQUIRE(rows > 0 && q_heads > 0 && kv_heads > 0 && q_heads % kv_heads == 0,
@@ -158,12 +177,12 @@ extern "C" int leone_attention_rows_kept(const void* q, void* out, const void* k
         attention_rows_kernel<float><<<grid, kRowThreads, 0, stream>>>(
             static_cast<const float*>(q), static_cast<float*>(out), static_cast<const float*>(k_pool),
             static_cast<const float*>(v_pool), positions, row_entry, block_table, max_blocks, q_heads, kv_heads,
-            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride, keep_first, gate_each);
+            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride, keep_first, gate_each, slopes, temp_coef, temp_every);
     else
         attention_rows_kernel<bf16_t><<<grid, kRowThreads, 0, stream>>>(
             static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_pool),
             static_cast<const bf16_t*>(v_pool), positions, row_entry, block_table, max_blocks, q_heads, kv_heads,
-            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride, keep_first, gate_each);
+            head_dim, v_dim, page_tokens, scale, window, gate, gate_stride, keep_first, gate_each, slopes, temp_coef, temp_every);
     LEONE_LAUNCH_CHECK("attention_rows");
     return 0;
 }

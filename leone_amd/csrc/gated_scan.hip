@@ -4,6 +4,10 @@
 //                 S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T,   o_t = S_t^T q_t,   q_t = act(q_pre_t)
 //                 (1 - f_t is taken as (1 - lower) * sigmoid(-(pre_t + bias)), which keeps its digits where f_t
 //                 is close to 1)
+//   state_space_scan   the same walk for a state-space layer whose decay is one number a head and row:
+//                 dt_t = softplus(pre_t + bias),  f_t = exp(-exp(rate_log) * dt_t)  for every key channel of the head,
+//                 S_t = f_t S_(t-1) + (dt_t B_t) x_t^T,   o_t = S_t^T C_t + skip * x_t
+//                 with B and C shared by the heads of a group (head h reads group h / (heads / groups))
 //   gated_chain   chains the end states of chunks that were walked side by side (see below).
 //
 // The layout is that of the other matrix-memory recurrences: a workgroup of four waves owns a run of columns of one
@@ -52,9 +56,18 @@ struct GatedScanArgs {
     float* gate_product;            // [segments, heads, dim]: the product of f_t over the segment's rows, or null
     float* out;                     // [rows, heads, vdim]
     int heads, dim, vdim;
+    // the state-space form: q (the read vector C) and the write vector B come in qk_heads groups of dim columns
+    // (B's group 0 at k_off), the step size's pre-activation at step[row * step_stride + step_off + head]
+    int qk_heads, k_off;
+    const float* step;
+    long step_stride;
+    int step_off;
+    AnyVec step_bias, rate_log, skip;   // [heads] each
 };
 
-template <bool kTrack>
+enum GsKind : int { kGsGated = 0, kGsStateSpace = 1 };
+
+template <bool kTrack, int kKind>
 __global__ void __launch_bounds__(kGsThreads) gated_scan_kernel(GatedScanArgs p, int groups) {
     extern __shared__ __align__(16) float gs_lds[];
     const int dkp = groups * kGsLaneRows;
@@ -71,6 +84,9 @@ __global__ void __launch_bounds__(kGsThreads) gated_scan_kernel(GatedScanArgs p,
         col[c] = ((blockIdx.z * (kGsThreads / kWave) + tid / kWave) * kGsLaneCols + c) * per_wave + lane % per_wave;
     const int first = seg.first, n = seg.end - seg.first;
     const int ch0 = part * kGsLaneRows;
+    const int shared_head = kKind == kGsStateSpace ? head / (p.heads / p.qk_heads) : head;
+    const float skip = kKind == kGsStateSpace ? load_any(p.skip, head) : 0.f;
+    const float rate = kKind == kGsStateSpace ? expf(load_any(p.rate_log, head)) : 0.f;
     const float* from = seg.in < 0 ? nullptr : p.state_in + seg.in * p.in_stride + static_cast<long>(head) * p.dim * p.vdim;
 
     float S[kGsLaneCols][kGsLaneRows];
@@ -90,7 +106,17 @@ __global__ void __launch_bounds__(kGsThreads) gated_scan_kernel(GatedScanArgs p,
         for (int idx = tid; idx < here * dkp; idx += kGsThreads) {
             const int t = idx / dkp, i = idx % dkp;
             float qv = 0.f, fv = 1.f, kv = 0.f;
-            if (i < p.dim) {
+            if (kKind == kGsStateSpace) {
+                if (i < p.dim) {
+                    const long r = first + t0 + t;
+                    const float* base = p.proj + r * p.stride;
+                    qv = base[p.q_off + shared_head * p.dim + i];
+                    const float z = p.step[r * p.step_stride + p.step_off + head] + load_any(p.step_bias, head);
+                    const float dt = z > 20.f ? z : log1pf(expf(z));
+                    fv = expf(-rate * dt);
+                    kv = p.no_input ? 0.f : dt * base[p.k_off + shared_head * p.dim + i];
+                }
+            } else if (i < p.dim) {
                 const float* base = p.proj + static_cast<long>(first + t0 + t) * p.stride;
                 const float qp = base[p.q_off + head * p.dim + i];
                 qv = p.q_silu ? qp / (1.0f + expf(-qp)) : qp;
@@ -132,7 +158,8 @@ __global__ void __launch_bounds__(kGsThreads) gated_scan_kernel(GatedScanArgs p,
                     for (int off = per_wave; off < kWave; off <<= 1) acc[c] += __shfl_xor(acc[c], off, kWave);
                     if (part == 0 && col[c] < p.vdim) {
                         float* dst = p.out + (row * p.heads + head) * p.vdim + col[c];
-                        *dst = p.accumulate ? *dst + acc[c] : acc[c];
+                        const float read = kKind == kGsStateSpace ? fmaf(skip, v[c], acc[c]) : acc[c];
+                        *dst = p.accumulate ? *dst + read : read;
                     }
                 }
             }
@@ -203,14 +230,52 @@ extern "C" int leone_gated_scan(const float* proj, long stride, int q_off, int f
                   stride >= v_off + heads * vdim, "gated_scan: the projection's rows of %ld do not hold the named columns", stride);
     GatedScanArgs a{proj, stride, q_off, f_off, v_off, AnyVec{f_bias, vec_dtype}, AnyVec{lower, vec_dtype}, q_silu, no_input,
                     accumulate, reinterpret_cast<const GsSegment*>(segments), state_in, in_stride, state_out, out_stride,
-                    gate_product, out, heads, dim, vdim};
+                    gate_product, out, heads, dim, vdim, heads, 0, nullptr, 0, 0, AnyVec{nullptr, vec_dtype},
+                    AnyVec{nullptr, vec_dtype}, AnyVec{nullptr, vec_dtype}};
     const int groups = gs_lane_groups(dim);
     const int per_block = (kGsThreads / kWave) * (kWave / groups) * kGsLaneCols;
     const dim3 grid(n_segments, heads, ceil_div(vdim, per_block));
     const size_t shared = 3 * kGsTokens * groups * kGsLaneRows * sizeof(float);
-    if (gate_product) gated_scan_kernel<true><<<grid, kGsThreads, shared, stream>>>(a, groups);
-    else gated_scan_kernel<false><<<grid, kGsThreads, shared, stream>>>(a, groups);
+    if (gate_product) gated_scan_kernel<true, kGsGated><<<grid, kGsThreads, shared, stream>>>(a, groups);
+    else gated_scan_kernel<false, kGsGated><<<grid, kGsThreads, shared, stream>>>(a, groups);
     LEONE_LAUNCH_CHECK("gated_scan");
+    return 0;
+}
+
+// The state-space form.  xbc float [rows, stride] holds x (heads * vdim columns from x_off), B and C (groups * dim columns
+// each from b_off and c_off); step float [rows, step_stride] the step sizes' pre-activations (heads columns from step_off);
+// step_bias, rate_log, skip [heads] of vec_dtype.  States, segments, products and out as for leone_gated_scan (dim is the
+// state size a head, the rows of S).
+extern "C" int leone_state_space_scan(const float* xbc, long stride, int x_off, int b_off, int c_off, int groups_bc,
+                                      const float* step, long step_stride, int step_off, const void* step_bias,
+                                      const void* rate_log, const void* skip, int vec_dtype, int no_input, int accumulate,
+                                      const int* segments, int n_segments, const float* state_in, long in_stride,
+                                      float* state_out, long out_stride, float* gate_product, float* out, int heads, int dim,
+                                      int vdim, hipStream_t stream) {
+    LEONE_REQUIRE(xbc && step && step_bias && rate_log && skip && segments && out, "state_space_scan: null pointer");
+    LEONE_REQUIRE(vec_dtype == kF32 || vec_dtype == kBF16, "state_space_scan: unknown element type");
+    LEONE_REQUIRE(n_segments > 0 && heads > 0 && heads <= 65535 && dim > 0 && vdim > 0, "state_space_scan: %d segments, %d heads of %d x %d",
+                  n_segments, heads, dim, vdim);
+    LEONE_REQUIRE(groups_bc > 0 && heads % groups_bc == 0, "state_space_scan: %d heads do not share %d groups evenly", heads, groups_bc);
+    LEONE_REQUIRE(dim <= kGsMaxDim, "state_space_scan: states of %d rows a head, the kernel takes up to %d", dim, kGsMaxDim);
+    const long per_slot = static_cast<long>(heads) * dim * vdim;
+    LEONE_REQUIRE((!state_in || in_stride >= per_slot) && (!state_out || out_stride >= per_slot),
+                  "state_space_scan: states of %ld floats do not fit", per_slot);
+    LEONE_REQUIRE(x_off >= 0 && b_off >= 0 && c_off >= 0 && stride >= x_off + heads * vdim && stride >= b_off + groups_bc * dim &&
+                  stride >= c_off + groups_bc * dim, "state_space_scan: rows of %ld do not hold the named columns", stride);
+    LEONE_REQUIRE(step_off >= 0 && step_stride >= step_off + heads, "state_space_scan: rows of %ld do not hold %d step sizes",
+                  step_stride, heads);
+    GatedScanArgs a{xbc, stride, c_off, 0, x_off, AnyVec{nullptr, vec_dtype}, AnyVec{nullptr, vec_dtype}, 0, no_input,
+                    accumulate, reinterpret_cast<const GsSegment*>(segments), state_in, in_stride, state_out, out_stride,
+                    gate_product, out, heads, dim, vdim, groups_bc, b_off, step, step_stride, step_off,
+                    AnyVec{step_bias, vec_dtype}, AnyVec{rate_log, vec_dtype}, AnyVec{skip, vec_dtype}};
+    const int groups = gs_lane_groups(dim);
+    const int per_block = (kGsThreads / kWave) * (kWave / groups) * kGsLaneCols;
+    const dim3 grid(n_segments, heads, ceil_div(vdim, per_block));
+    const size_t shared = 3 * kGsTokens * groups * kGsLaneRows * sizeof(float);
+    if (gate_product) gated_scan_kernel<true, kGsStateSpace><<<grid, kGsThreads, shared, stream>>>(a, groups);
+    else gated_scan_kernel<false, kGsStateSpace><<<grid, kGsThreads, shared, stream>>>(a, groups);
+    LEONE_LAUNCH_CHECK("state_space_scan");
     return 0;
 }
 

@@ -130,7 +130,7 @@ constexpr int kConvRows = 8;     // consecutive rows a workgroup takes in a step
 
 template <typename TIn, typename TOut>
 __global__ void causal_conv_kernel(const TIn* __restrict__ in, long in_stride, TOut* __restrict__ out, long out_stride,
-                                   AnyVec w, const float* __restrict__ state, const int* __restrict__ positions,
+                                   AnyVec w, AnyVec bias, const float* __restrict__ state, const int* __restrict__ positions,
                                    const int* __restrict__ row_entry, const int* __restrict__ entry_slots, int rows,
                                    int channels, int taps, int add_input, int act, float* __restrict__ own_state, int per_block) {
     __shared__ int s_inside[kConvRows], s_pos[kConvRows], s_slot[kConvRows];
@@ -161,6 +161,7 @@ __global__ void causal_conv_kernel(const TIn* __restrict__ in, long in_stride, T
         }
         const float now = to_float(in[static_cast<long>(r) * in_stride + c]);
         if (add_input) acc += now;
+        if (bias.ptr) acc += load_any(bias, c);
         out[static_cast<long>(r) * out_stride + c] = from_float<TOut>(activate(acc, act));
         if (own_state) {      // a step of single rows, every row another request: this thread alone touches (slot, channel)
             float* keep = own_state + (static_cast<long>(s_slot[k]) * (taps - 1)) * channels + c;
@@ -195,7 +196,7 @@ __global__ void causal_conv_state_kernel(const TIn* __restrict__ in, long in_str
 template <typename TOut>
 __global__ void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ dot, const float* __restrict__ top,
                                       AnyVec gain, int gain_per_head, const float* __restrict__ gate, long gate_stride,
-                                      int act, float eps, TOut* __restrict__ out, int heads, int vdim) {
+                                      int act, float eps, TOut* __restrict__ out, int heads, int vdim, int gate_first) {
     const int row = blockIdx.x;
     const int head = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
     const int lane = threadIdx.x % kWave;
@@ -204,17 +205,23 @@ __global__ void head_norm_gate_kernel(const float* __restrict__ o, const float* 
     const float* src = o + at * vdim;
     float under = 1.f;
     if (dot) under = fmaxf(fabsf(dot[at]), expf(-top[at])) + 1e-6f;
+    const float* gate_row = gate ? gate + static_cast<long>(row) * gate_stride + static_cast<long>(head) * vdim : nullptr;
+    // with gate_first the gate multiplies ahead of the norm, and the root mean square is that of the gated values
+    auto fetch = [&](int j) {
+        const float v = src[j] / under;
+        return (gate_first && gate_row) ? v * activate(gate_row[j], act) : v;
+    };
     constexpr int kKept = 8;                                   // values a lane keeps between the two passes
     float kept[kKept];
     float ss = 0.f;
 #pragma unroll
     for (int n = 0; n < kKept; ++n) {
         const int j = lane + n * kWave;
-        kept[n] = j < vdim ? src[j] / under : 0.f;
+        kept[n] = j < vdim ? fetch(j) : 0.f;
         ss = fmaf(kept[n], kept[n], ss);
     }
     for (int j = lane + kKept * kWave; j < vdim; j += kWave) {
-        const float v = src[j] / under;
+        const float v = fetch(j);
         ss = fmaf(v, v, ss);
     }
     const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps);
@@ -222,13 +229,13 @@ __global__ void head_norm_gate_kernel(const float* __restrict__ o, const float* 
     auto finish = [&](int j, float v) {
         v *= inv;
         if (gain.ptr) v *= load_any(gain, gain_per_head ? static_cast<long>(head) * vdim + j : j);
-        if (gate) v *= activate(gate[static_cast<long>(row) * gate_stride + static_cast<long>(head) * vdim + j], act);
+        if (gate_row && !gate_first) v *= activate(gate_row[j], act);
         dst[j] = from_float<TOut>(v);
     };
 #pragma unroll
     for (int n = 0; n < kKept; ++n)
         if (lane + n * kWave < vdim) finish(lane + n * kWave, kept[n]);
-    for (int j = lane + kKept * kWave; j < vdim; j += kWave) finish(j, src[j] / under);
+    for (int j = lane + kKept * kWave; j < vdim; j += kWave) finish(j, fetch(j));
 }
 
 constexpr int kMaxBranches = 4;
@@ -253,6 +260,16 @@ rms_mix_kernel(Branches in, int branches, float eps, float scale, float* __restr
         float total = 0.f;
         for (int b = 0; b < branches; ++b) total += in.rows[b][row * hidden + i] * inv[b] * load_any(in.gain[b], i);
         out[row * hidden + i] = total * scale;
+    }
+}
+
+// out = sum_b weight_b * branch_b, nothing normed.
+__global__ void weighted_mix_kernel(Branches in, int branches, float w0, float w1, float w2, float w3, float* __restrict__ out, long n) {
+    const float weight[kMaxBranches] = {w0, w1, w2, w3};
+    for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < n; i += static_cast<long>(gridDim.x) * blockDim.x) {
+        float total = 0.f;
+        for (int b = 0; b < branches; ++b) total = fmaf(weight[b], in.rows[b][i], total);
+        out[i] = total;
     }
 }
 
@@ -327,6 +344,17 @@ extern "C" int leone_causal_conv(const void* in, int in_dtype, long in_stride, v
                                  const void* w, int w_dtype, float* state, int write_state, const int* spans, int entries,
                                  const int* positions, const int* row_entry, const int* entry_slots, int rows,
                                  int channels, int taps, int add_input, int act, int single_rows, hipStream_t stream) {
+    return leone_causal_conv_biased(in, in_dtype, in_stride, out, out_dtype, out_stride, w, nullptr, w_dtype, state, write_state,
+                                    spans, entries, positions, row_entry, entry_slots, rows, channels, taps, add_input, act,
+                                    single_rows, stream);
+}
+
+// bias: one value a channel ([channels], of the filters' type) added to the filter's sum ahead of the activation; may be null.
+extern "C" int leone_causal_conv_biased(const void* in, int in_dtype, long in_stride, void* out, int out_dtype, long out_stride,
+                                        const void* w, const void* bias, int w_dtype, float* state, int write_state,
+                                        const int* spans, int entries, const int* positions, const int* row_entry,
+                                        const int* entry_slots, int rows, int channels, int taps, int add_input, int act,
+                                        int single_rows, hipStream_t stream) {
     LEONE_REQUIRE(in && out && w && state && positions && row_entry && entry_slots, "causal_conv: null pointer");
     LEONE_REQUIRE(known(in_dtype) && known(out_dtype) && known(w_dtype), "causal_conv: unknown element type");
     LEONE_REQUIRE(rows > 0 && channels > 0 && ceil_div(channels, 256) <= 65535 && in_stride >= channels && out_stride >= channels,
@@ -336,11 +364,12 @@ extern "C" int leone_causal_conv(const void* in, int in_dtype, long in_stride, v
     LEONE_REQUIRE(!write_state || single_rows || (spans && entries > 0 && entries <= 65535),
                   "causal_conv: the state's update needs the entries' spans");
     const AnyVec vw{w, w_dtype};
+    const AnyVec vbias{bias, w_dtype};
     const int per_block = rows >= kNormManyRows ? kConvRows : 1;
     const dim3 grid(ceil_div(rows, per_block), ceil_div(channels, 256));
 #define LEONE_CONV(TIN, TOUT)                                                                                         \
     causal_conv_kernel<TIN, TOUT><<<grid, 256, 0, stream>>>(static_cast<const TIN*>(in), in_stride, static_cast<TOUT*>(out), \
-                                                            out_stride, vw, state, positions, row_entry, entry_slots, \
+                                                            out_stride, vw, vbias, state, positions, row_entry, entry_slots, \
                                                             rows, channels, taps, add_input, act,                    \
                                                             (write_state && single_rows) ? state : nullptr, per_block)
     if (in_dtype == kF32 && out_dtype == kF32) LEONE_CONV(float, float);
@@ -365,6 +394,15 @@ extern "C" int leone_causal_conv(const void* in, int in_dtype, long in_stride, v
 extern "C" int leone_head_norm_gate(const float* o, const float* dot, const float* top, const void* gain, int gain_dtype,
                                     int gain_per_head, const float* gate, long gate_stride, int act, float eps, void* out,
                                     int out_dtype, int rows, int heads, int vdim, hipStream_t stream) {
+    return leone_head_norm_gate_ordered(o, dot, top, gain, gain_dtype, gain_per_head, gate, gate_stride, act, 0, eps, out,
+                                        out_dtype, rows, heads, vdim, stream);
+}
+
+// gate_first: the gate multiplies ahead of the norm (the root mean square is taken of the gated values) instead of behind it.
+extern "C" int leone_head_norm_gate_ordered(const float* o, const float* dot, const float* top, const void* gain, int gain_dtype,
+                                            int gain_per_head, const float* gate, long gate_stride, int act, int gate_first,
+                                            float eps, void* out, int out_dtype, int rows, int heads, int vdim,
+                                            hipStream_t stream) {
     LEONE_REQUIRE(o && out && rows > 0 && heads > 0 && vdim > 0, "head_norm_gate: needs read-outs and positive sizes");
     LEONE_REQUIRE(known(out_dtype) && (!gain || known(gain_dtype)), "head_norm_gate: unknown element type");
     LEONE_REQUIRE((dot == nullptr) == (top == nullptr), "head_norm_gate: the denominator's two parts come together");
@@ -374,10 +412,10 @@ extern "C" int leone_head_norm_gate(const float* o, const float* dot, const floa
     const dim3 grid(rows, ceil_div(heads, 4));
     if (out_dtype == kF32)
         head_norm_gate_kernel<float><<<grid, 4 * kWave, 0, stream>>>(o, dot, top, vg, gain_per_head, gate, gate_stride, act, eps,
-                                                                     static_cast<float*>(out), heads, vdim);
+                                                                     static_cast<float*>(out), heads, vdim, gate_first);
     else
         head_norm_gate_kernel<bf16_t><<<grid, 4 * kWave, 0, stream>>>(o, dot, top, vg, gain_per_head, gate, gate_stride, act, eps,
-                                                                      static_cast<bf16_t*>(out), heads, vdim);
+                                                                      static_cast<bf16_t*>(out), heads, vdim, gate_first);
     LEONE_LAUNCH_CHECK("head_norm_gate");
     return 0;
 }
@@ -396,6 +434,23 @@ extern "C" int leone_rms_mix(const float* const* branch_rows, const void* const*
     if (rows >= kNormManyRows) rms_mix_kernel<kNormThreadsMany><<<rows, kNormThreadsMany, 0, stream>>>(in, branches, eps, scale, out, hidden);
     else rms_mix_kernel<kNormThreadsFew><<<rows, kNormThreadsFew, 0, stream>>>(in, branches, eps, scale, out, hidden);
     LEONE_LAUNCH_CHECK("rms_mix");
+    return 0;
+}
+
+extern "C" int leone_weighted_mix(const float* const* branch_rows, const float* weights, int branches, float* out, long n,
+                                  hipStream_t stream) {
+    LEONE_REQUIRE(branch_rows && weights && out && n > 0, "weighted_mix: needs branches and a positive size");
+    LEONE_REQUIRE(branches >= 1 && branches <= kMaxBranches, "weighted_mix: %d branches, the kernel takes 1..%d", branches, kMaxBranches);
+    Branches in{};
+    float w[kMaxBranches] = {0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < branches; ++b) {
+        LEONE_REQUIRE(branch_rows[b], "weighted_mix: branch %d is missing", b);
+        in.rows[b] = branch_rows[b];
+        w[b] = weights[b];
+    }
+    const long blocks = (n + 255) / 256;
+    weighted_mix_kernel<<<static_cast<int>(blocks < 4096 ? blocks : 4096), 256, 0, stream>>>(in, branches, w[0], w[1], w[2], w[3], out, n);
+    LEONE_LAUNCH_CHECK("weighted_mix");
     return 0;
 }
 

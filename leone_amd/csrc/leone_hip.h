@@ -225,6 +225,30 @@ int leone_causal_conv(const void* in, int in_dtype, long in_stride, void* out, i
 int leone_head_norm_gate(const float* o, const float* dot, const float* top, const void* gain, int gain_dtype,
                          int gain_per_head, const float* gate, long gate_stride, int act, float eps, void* out,
                          int out_dtype, int rows, int heads, int vdim, hipStream_t stream);
+// Projections with biases (see biased.hip).  bias_span_norm, in place on float rows [rows, stride]: the first `biased` columns
+// get bias[c] (may be null) and, with round_bf16, bfloat16's rounding; then span s (columns offsets[s] .. + widths[s]) is
+// divided by its root mean square over the whole span and multiplied by gains[s] ([widths[s]]).  offsets, widths and gains
+// are host arrays.
+int leone_bias_span_norm(float* rows_at, long stride, int rows, const void* bias, int bias_dtype, int biased, int round_bf16,
+                         const int* offsets, const int* widths, const void* const* gains, int gain_dtype, int n_spans,
+                         float eps, hipStream_t stream);
+// out[r, c] = act(gate_up[r, c] + bias[c]) * (gate_up[r, ffn + c] + bias[ffn + c]); act 0 silu, 1 the tanh form of gelu.
+int leone_bias_glu(const void* gate_up, int in_dtype, const void* bias, int bias_dtype, void* out, int out_dtype, int rows,
+                   int ffn, int act, hipStream_t stream);
+// x[r, c] += bias[c] in place, x float [rows, width].
+int leone_add_bias(float* x, const void* bias, int bias_dtype, int rows, int width, hipStream_t stream);
+// leone_causal_conv with a bias a channel (of the filters' type, may be null) added ahead of the activation.
+int leone_causal_conv_biased(const void* in, int in_dtype, long in_stride, void* out, int out_dtype, long out_stride,
+                             const void* w, const void* bias, int w_dtype, float* state, int write_state, const int* spans,
+                             int entries, const int* positions, const int* row_entry, const int* entry_slots, int rows,
+                             int channels, int taps, int add_input, int act, int single_rows, hipStream_t stream);
+// leone_head_norm_gate with the gate ahead of the norm if gate_first.
+int leone_head_norm_gate_ordered(const float* o, const float* dot, const float* top, const void* gain, int gain_dtype,
+                                 int gain_per_head, const float* gate, long gate_stride, int act, int gate_first, float eps,
+                                 void* out, int out_dtype, int rows, int heads, int vdim, hipStream_t stream);
+// out = sum over branches of weights[b] * branch (host floats; n elements each), nothing normed.
+int leone_weighted_mix(const float* const* branch_rows, const float* weights, int branches, float* out, long n,
+                       hipStream_t stream);
 // out = scale * sum over branches of rms(branch) * gain.
 int leone_rms_mix(const float* const* branch_rows, const void* const* gains, int gain_dtype, int branches, float eps,
                   float scale, float* out, int rows, int hidden, hipStream_t stream);
@@ -272,6 +296,14 @@ int leone_attention_rows_kept(const void* q, void* out, const void* k_pool, cons
                               int rows, int q_heads, int kv_heads, int head_dim, int v_dim, int page_tokens,
                               float scale, int window, const float* gate, long gate_stride, int keep_first,
                               int gate_each, hipStream_t stream);
+// leone_attention_rows_kept with a distance bias (slopes float [q_heads] or null: head h's score at distance d is lowered by
+// slopes[h] * d) and a query factor that grows with the position (temp_every > 0: 1 + temp_coef * ln(floor((pos + 1) /
+// temp_every) + 1)).
+int leone_attention_rows_biased(const void* q, void* out, const void* k_pool, const void* v_pool, int dtype,
+                                const int* positions, const int* row_entry, const int* block_table, int max_blocks,
+                                int rows, int q_heads, int kv_heads, int head_dim, int v_dim, int page_tokens,
+                                float scale, int window, const float* gate, long gate_stride, int keep_first,
+                                int gate_each, const float* slopes, float temp_coef, int temp_every, hipStream_t stream);
 // leone_attention_decode with the keys at positions below keep_first kept in sight of a windowed layer.
 int leone_attention_decode_kept(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
                                 const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
@@ -312,6 +344,13 @@ int leone_gated_scan(const float* proj, long stride, int q_off, int f_off, int v
                      int vec_dtype, int q_silu, int no_input, int accumulate, const int* segments, int n_segments,
                      const float* state_in, long in_stride, float* state_out, long out_stride, float* gate_product, float* out,
                      int heads, int dim, int vdim, hipStream_t stream);
+// The same walk for a state-space layer: S <- exp(-exp(rate_log) dt) S + (dt B) x^T, o = S^T C + skip x, dt =
+// softplus(step + step_bias); B and C in groups_bc groups shared by neighbouring heads.  Chunks chain through leone_gated_chain.
+int leone_state_space_scan(const float* xbc, long stride, int x_off, int b_off, int c_off, int groups_bc, const float* step,
+                           long step_stride, int step_off, const void* step_bias, const void* rate_log, const void* skip,
+                           int vec_dtype, int no_input, int accumulate, const int* segments, int n_segments,
+                           const float* state_in, long in_stride, float* state_out, long out_stride, float* gate_product,
+                           float* out, int heads, int dim, int vdim, hipStream_t stream);
 int leone_gated_chain(const int* links, int n_links, float* work, long work_stride, const float* product, float* state,
                       long slot_stride, int heads, int dim, int vdim, int write_state, hipStream_t stream);
 // Attention through a latent that all heads share (see latent.hip).

@@ -297,10 +297,13 @@ def _strided_rows(t: Optional[torch.Tensor], what: str, rows: int, columns: int,
 def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
                    row_entry: torch.Tensor, block_table: torch.Tensor, q_heads: int, scale: float,
                    window: int = 0, out: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
-                   keep_first: int = 0, gate_each: bool = False) -> torch.Tensor:
+                   keep_first: int = 0, gate_each: bool = False, slopes: Optional[torch.Tensor] = None,
+                   query_factor: Optional[tuple] = None) -> torch.Tensor:
     """Each query row attends its request's cached keys up to its own position (the last ``window`` of them,
     and, whatever the window, those at positions below ``keep_first``).  The result has the values'
-    size a head.  ``gate``: float32 ``[rows, >= q_heads]`` (a view into a wider row is fine, unit stride along the
+    size a head.  ``slopes`` float32 ``[q_heads]``: head h's score for the key at distance d is lowered by
+    slopes[h] * d.  ``query_factor`` = (coef, every): the queries of a row at position p count times
+    1 + coef * ln(floor((p + 1) / every) + 1).  ``gate``: float32 ``[rows, >= q_heads]`` (a view into a wider row is fine, unit stride along the
     heads): head h of row r is multiplied by sigmoid(gate[r, h]); with ``gate_each`` the gate holds a value for
     every element of the result, ``[rows, >= q_heads * value_dim]``."""
     rows = q.shape[0]
@@ -310,12 +313,14 @@ def attention_rows(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, 
     if out is None:
         out = torch.empty((rows, q_heads * value_dim), dtype=q.dtype, device=q.device)
     gate_at, gate_stride = _strided_rows(gate, "attention gate", rows, q_heads * value_dim if gate_each else q_heads)
-    call("leone_attention_rows_kept", _dev(q, "attention q"), _dev(out, "attention out", q.dtype, (rows, q_heads * value_dim)),
+    coef, every = query_factor if query_factor is not None else (0.0, 0)
+    call("leone_attention_rows_biased", _dev(q, "attention q"), _dev(out, "attention out", q.dtype, (rows, q_heads * value_dim)),
          _dev(k_pool, "k pool", q.dtype), _dev(v_pool, "v pool", q.dtype), _code(q, "attention q"),
          _dev(positions, "positions", torch.int32, (rows,)), _dev(row_entry, "row map", torch.int32, (rows,)),
          _dev(block_table, "block table", torch.int32), block_table.shape[1], rows, q_heads, kv_heads, head_dim,
          value_dim, page_tokens, float(scale), int(window), gate_at, gate_stride, int(keep_first),
-         1 if (gate_each and gate is not None) else 0, _stream())
+         1 if (gate_each and gate is not None) else 0, _dev(slopes, "slopes", torch.float32, (q_heads,)), float(coef),
+         int(every), _stream())
     return out
 
 
@@ -1230,11 +1235,12 @@ def chunk_plan(step, chunk: int, chunked_from: int):
 
 
 def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, step, out_dtype: torch.dtype,
-                add_input: bool = False, activation: Optional[str] = None, write_state: bool = True) -> torch.Tensor:
-    """out[t, c] = (x[t, c] if ``add_input``) + sum_j weight[c, j] * x[t - (taps - 1) + j, c], then the
-    activation; rows before a portion come from ``state`` (float32 ``[slots, taps - 1, channels]``: a request's
+                add_input: bool = False, activation: Optional[str] = None, write_state: bool = True,
+                bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, c] = (x[t, c] if ``add_input``) + sum_j weight[c, j] * x[t - (taps - 1) + j, c] (+ ``bias[c]``), then
+    the activation; rows before a portion come from ``state`` (float32 ``[slots, taps - 1, channels]``: a request's
     last inputs), zeros before position 0.  ``x`` may be a column slice of wider rows.  Leaves the state
-    brought up to date unless told not to."""
+    brought up to date unless told not to.  ``bias`` ``[channels]`` comes in the filters' type."""
     rows, channels = x.shape
     taps = weight.shape[1]
     if tuple(weight.shape) != (channels, taps) or x.dim() != 2 or x.stride(1) != 1:
@@ -1243,11 +1249,14 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, step
         raise KernelError(f"causal_conv: state {tuple(state.shape)} is not [slots, {taps - 1}, {channels}] float32")
     if not x.is_cuda:
         raise KernelError("causal_conv: tensor is not on the GPU")
+    if bias is not None and bias.dtype != weight.dtype:
+        raise KernelError(f"causal_conv: a bias of {bias.dtype} beside filters of {weight.dtype}")
     out = torch.empty((rows, channels), dtype=out_dtype, device=x.device)
     spans = entry_spans(step)
     single_rows = bool(step.decode_only) and step.entry_slots.numel() == rows
-    call("leone_causal_conv", x.data_ptr(), _code(x, "conv input"), x.stride(0), _dev(out, "conv out"), _CODES[out_dtype],
-         channels, _dev(weight, "conv weight"), _code(weight, "conv weight"), _dev(state, "conv state"),
+    call("leone_causal_conv_biased", x.data_ptr(), _code(x, "conv input"), x.stride(0), _dev(out, "conv out"), _CODES[out_dtype],
+         channels, _dev(weight, "conv weight"), _dev(bias, "conv bias", None, (channels,)), _code(weight, "conv weight"),
+         _dev(state, "conv state"),
          1 if write_state else 0, _dev(spans, "spans"), spans.shape[0],
          _dev(step.positions, "positions", torch.int32, (rows,)), _dev(step.row_entry, "row map", torch.int32, (rows,)),
          _dev(step.entry_slots, "slots", torch.int32), rows, channels, taps, 1 if add_input else 0,
@@ -1257,11 +1266,13 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, step
 
 def head_norm_gate(o: torch.Tensor, heads: int, vdim: int, eps: float, out_dtype: torch.dtype,
                    gain: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
-                   activation: Optional[str] = None, denominator: Optional[tuple] = None) -> torch.Tensor:
+                   activation: Optional[str] = None, denominator: Optional[tuple] = None,
+                   gate_first: bool = False) -> torch.Tensor:
     """Head by head: o (float32 ``[rows, heads * vdim]``), divided by max(|dot|, exp(-top)) + 1e-6 if
     ``denominator`` = (dot, top) (float32 ``[rows, heads]``) comes, over its root mean square, times ``gain``
     (``[heads * vdim]``, or ``[vdim]`` shared by the heads), times activation(gate) (float32 rows of heads * vdim,
-    possibly a slice of wider rows)."""
+    possibly a slice of wider rows).  ``gate_first``: the gate multiplies ahead of the norm, so the root mean square
+    is that of the gated values.  A "head" is whatever run of ``vdim`` columns is normed by itself."""
     rows = o.shape[0]
     out = torch.empty((rows, heads * vdim), dtype=out_dtype, device=o.device)
     per_head = 0
@@ -1272,10 +1283,10 @@ def head_norm_gate(o: torch.Tensor, heads: int, vdim: int, eps: float, out_dtype
             raise KernelError(f"head_norm_gate: a gain of {gain.numel()} for {heads} heads of {vdim}")
     gate_at, gate_stride = _strided_rows(gate, "head_norm_gate gate", rows, heads * vdim)
     dot, top = denominator if denominator is not None else (None, None)
-    call("leone_head_norm_gate", _dev(o, "read-outs", torch.float32, (rows, heads * vdim)),
+    call("leone_head_norm_gate_ordered", _dev(o, "read-outs", torch.float32, (rows, heads * vdim)),
          _dev(dot, "dot", torch.float32, (rows, heads)), _dev(top, "top", torch.float32, (rows, heads)),
          _dev(gain, "gain"), _code(gain, "gain") if gain is not None else F32, per_head, gate_at, gate_stride,
-         ACTIVATIONS[activation], float(eps), _dev(out, "out"), _CODES[out_dtype], rows, heads, vdim, _stream())
+         ACTIVATIONS[activation], 1 if gate_first else 0, float(eps), _dev(out, "out"), _CODES[out_dtype], rows, heads, vdim, _stream())
     return out
 
 
@@ -1291,6 +1302,60 @@ def rms_mix(branches, gains, eps: float, scale: float) -> torch.Tensor:
     call("leone_rms_mix", ctypes.cast(row_ptrs, ctypes.c_void_p), ctypes.cast(gain_ptrs, ctypes.c_void_p),
          _code(gains[0], "branch gain"), len(branches), float(eps), float(scale), _dev(out, "out"), rows, hidden, _stream())
     return out
+
+
+def weighted_mix(branches, weights) -> torch.Tensor:
+    """sum_b weights[b] * branches[b]: float32 tensors of one shape, 1 to 4 of them, nothing normed."""
+    shape = tuple(branches[0].shape)
+    if len(branches) != len(weights) or not 1 <= len(branches) <= 4:
+        raise KernelError("weighted_mix: one weight for each of 1 to 4 branches")
+    out = torch.empty(shape, dtype=torch.float32, device=branches[0].device)
+    row_ptrs = (ctypes.c_void_p * len(branches))(*[_dev(b, "branch", torch.float32, shape) for b in branches])
+    factors = (ctypes.c_float * len(weights))(*[float(w) for w in weights])
+    call("leone_weighted_mix", ctypes.cast(row_ptrs, ctypes.c_void_p), ctypes.cast(factors, ctypes.c_void_p), len(branches),
+         _dev(out, "out"), out.numel(), _stream())
+    return out
+
+
+def bias_span_norm(rows: torch.Tensor, bias: Optional[torch.Tensor], spans, eps: float, round_to: Optional[torch.dtype] = None) -> torch.Tensor:
+    """In place on float32 ``rows`` ``[n, width]``: the first ``len(bias)`` columns get their bias (None: none) and, with
+    ``round_to`` bfloat16, that type's rounding (what a product kept in the engine's type would hold); then every span
+    ``(offset, width, gain)`` is divided by its root mean square over the whole span, eps inside the root, and multiplied
+    by ``gain`` ``[width]``.  Up to four spans that do not overlap."""
+    n, width = rows.shape
+    spans = list(spans)
+    gains = [g for _, _, g in spans]
+    if len({g.dtype for g in gains}) > 1:
+        raise KernelError("bias_span_norm: the gains must come in one type")
+    biased = bias.numel() if bias is not None else (width if round_to == torch.bfloat16 else 0)
+    offsets = (ctypes.c_int * max(len(spans), 1))(*[int(o) for o, _, _ in spans])
+    widths = (ctypes.c_int * max(len(spans), 1))(*[int(w) for _, w, _ in spans])
+    gain_ptrs = (ctypes.c_void_p * max(len(spans), 1))(*[_dev(g, "span gain", None, (int(w),)) for _, w, g in spans])
+    call("leone_bias_span_norm", _dev(rows, "rows", torch.float32), width, n, _dev(bias, "bias"),
+         _code(bias, "bias") if bias is not None else F32, biased, 1 if round_to == torch.bfloat16 else 0,
+         ctypes.cast(offsets, ctypes.c_void_p), ctypes.cast(widths, ctypes.c_void_p), ctypes.cast(gain_ptrs, ctypes.c_void_p),
+         _code(gains[0], "span gain") if gains else F32, len(spans), float(eps), _stream())
+    return rows
+
+
+def bias_glu(gate_up: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype, activation: str = "silu") -> torch.Tensor:
+    """act(gate + b_gate) * (up + b_up) from rows ``[gate | up]`` ``[n, 2 ff]`` (one half behind the other) and a bias of
+    the same order ``[2 ff]`` (None: none) -> ``[n, ff]`` in ``out_dtype``."""
+    n, both = gate_up.shape
+    if both % 2:
+        raise KernelError(f"bias_glu: rows of {both} are no [gate | up]")
+    out = torch.empty((n, both // 2), dtype=out_dtype, device=gate_up.device)
+    call("leone_bias_glu", _dev(gate_up, "gate and up"), _code(gate_up, "gate and up"), _dev(bias, "bias", None, (both,)),
+         _code(bias, "bias") if bias is not None else F32, _dev(out, "out"), _CODES[out_dtype], n, both // 2,
+         _gate_code(activation), _stream())
+    return out
+
+
+def add_bias(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """x[r, c] += bias[c], in place on float32 rows."""
+    n, width = x.shape
+    call("leone_add_bias", _dev(x, "rows", torch.float32), _dev(bias, "bias", None, (width,)), _code(bias, "bias"), n, width, _stream())
+    return x
 
 
 def relu_squared(x: torch.Tensor) -> torch.Tensor:
@@ -1661,6 +1726,55 @@ def gated_scan(proj: torch.Tensor, columns: dict, f_bias: torch.Tensor, lower: t
     return out
 
 
+def state_space_scan(xbc: torch.Tensor, columns: dict, groups: int, step_size: torch.Tensor, step_bias: torch.Tensor,
+                     rate_log: torch.Tensor, skip: torch.Tensor, state: torch.Tensor, step, heads: int, dim: int, vdim: int,
+                     write_state: bool = True) -> torch.Tensor:
+    """A state-space layer's recurrence over every entry's rows: per head, with dt = softplus(pre + step_bias),
+    S <- exp(-exp(rate_log) dt) S + (dt B) x^T (S is ``dim`` x ``vdim``), o = S^T C + skip x.  ``xbc`` float32
+    ``[rows, width]`` holds x (``heads * vdim`` columns from ``columns["x"]``), B and C (``groups * dim`` columns each from
+    "b" and "c"; head h reads group h // (heads / groups)); ``step_size`` float32 ``[rows, >= heads]`` the step sizes'
+    pre-activations (a slice of wider rows is fine); ``step_bias``, ``rate_log``, ``skip`` ``[heads]`` of one type;
+    ``state`` float32 ``[slots, heads, dim * vdim]``.  Returns o float32 ``[rows, heads * vdim]``.  Long portions are walked
+    in chunks side by side, as in ``gated_scan``, chained by the product of the chunk's decays."""
+    rows, width = xbc.shape
+    if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (heads, dim * vdim) or not state.is_contiguous():
+        raise KernelError(f"state_space_scan: state {tuple(state.shape)} is not [slots, {heads}, {dim * vdim}] float32")
+    if len({step_bias.dtype, rate_log.dtype, skip.dtype}) != 1:
+        raise KernelError("state_space_scan: the step bias, the rates' logarithms and the skip weights must share one type")
+    if groups <= 0 or heads % groups:
+        raise KernelError(f"state_space_scan: {heads} heads do not share {groups} groups evenly")
+    step_at, step_stride = _strided_rows(step_size, "step sizes", rows, heads)
+    spans = entry_spans(step)
+    device = xbc.device
+    out = torch.empty((rows, heads * vdim), dtype=torch.float32, device=device)
+
+    def walk(segments, state_in, state_out, no_input=False, accumulate=False, product=None):
+        call("leone_state_space_scan", _dev(xbc, "x, B and C", torch.float32), width, columns["x"], columns["b"], columns["c"],
+             groups, step_at, step_stride, 0, _dev(step_bias, "step bias", None, (heads,)),
+             _dev(rate_log, "rate logarithms", None, (heads,)), _dev(skip, "skip weights", None, (heads,)),
+             _code(step_bias, "step bias"), 1 if no_input else 0, 1 if accumulate else 0,
+             _dev(segments, "segments", torch.int32), segments.shape[0],
+             _dev(state_in, "state read"), state_in.stride(0) if state_in is not None else 0,
+             _dev(state_out, "state written"), state_out.stride(0) if state_out is not None else 0,
+             _dev(product, "decay products"), _dev(out, "out"), heads, dim, vdim, _stream())
+
+    plan = chunk_plan(step, *GATED_CHUNKS)
+    if plan is None:
+        walk(spans, state, state if write_state else None)
+    else:
+        chunks = plan["chunks"]
+        work = torch.empty((chunks.shape[0], heads, dim * vdim), dtype=torch.float32, device=device)
+        product = torch.empty((chunks.shape[0], heads, dim), dtype=torch.float32, device=device)
+        walk(chunks, None, work, product=product)
+        call("leone_gated_chain", _dev(plan["links"], "links", torch.int32), plan["links"].shape[0], _dev(work, "work"),
+             work.stride(0), _dev(product, "decay products"), _dev(state, "state"), state.stride(0), heads, dim, vdim,
+             1 if write_state else 0, _stream())
+        walk(plan["again"], work, None, no_input=True, accumulate=True)
+        if plan["short"].shape[0]:
+            walk(plan["short"], state, state if write_state else None)
+    return out
+
+
 def _rotation_tables(what: str, part: int, cos, sin):
     """(address of cos, of sin, pairs, table positions) of a rotation of neighbouring pairs on the first elements of a
     part of ``part`` elements."""
@@ -1727,7 +1841,8 @@ def head_product(x: torch.Tensor, weight: torch.Tensor, heads: int, out_dtype: t
                  cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
                  positions: Optional[torch.Tensor] = None) -> torch.Tensor:
     """A product a head: ``x`` float32 ``[rows, heads * (inner + tail)]``, ``weight`` ``[heads, inner, outer]`` ->
-    ``[rows, heads * (outer + tail)]`` in ``out_dtype`` with y[r, h, :outer] = x[r, h, :inner] weight[h].  The ``tail``
+    ``[rows, heads * (outer + tail)]`` in ``out_dtype`` with y[r, h, :outer] = x[r, h, :inner] weight[h] (``x`` may be a
+    column slice of wider rows).  The ``tail``
     elements behind a head's inner ones are handed on behind its outer ones, rotated in neighbouring pairs by the
     row's position if tables come.  Many rows of a bfloat16 model go through the library's batched product (the rows
     rounded to bfloat16, float accumulation); the kernel then hands on the tails alone."""
@@ -1748,7 +1863,8 @@ def head_product(x: torch.Tensor, weight: torch.Tensor, heads: int, out_dtype: t
             out.view(rows, heads, outer + tail)[:, :, :outer].copy_(y.transpose(0, 1))
         if not tail:
             return out
-    call("leone_head_product", _dev(x, "head rows", torch.float32), x.shape[1], inner + tail,
+    x_at, x_stride = _strided_rows(x, "head rows", rows, x.shape[1])
+    call("leone_head_product", x_at, x_stride, inner + tail,
          0 if library else _dev(weight, "head matrices"), _code(weight, "head matrices"), _dev(out, "head results"),
          _CODES[out_dtype], out.shape[1], outer + tail, rows, heads,
          inner, outer, int(tail), cos_at, sin_at, pairs, table_positions,

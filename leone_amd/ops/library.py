@@ -58,6 +58,17 @@ _PROTOTYPES = {
     "leone_causal_conv": [P, c_int, ctypes.c_long, P, c_int, ctypes.c_long, P, c_int, P, c_int, P, c_int, P, P, P, c_int,
                           c_int, c_int, c_int, c_int, c_int, P],
     "leone_head_norm_gate": [P, P, P, P, c_int, c_int, P, ctypes.c_long, c_int, c_float, P, c_int, c_int, c_int, c_int, P],
+    "leone_head_norm_gate_ordered": [P, P, P, P, c_int, c_int, P, ctypes.c_long, c_int, c_int, c_float, P, c_int, c_int, c_int, c_int, P],
+    "leone_weighted_mix": [P, P, c_int, P, ctypes.c_long, P],
+    "leone_causal_conv_biased": [P, c_int, ctypes.c_long, P, c_int, ctypes.c_long, P, P, c_int, P, c_int, P, c_int, P, P, P, c_int,
+                                 c_int, c_int, c_int, c_int, c_int, P],
+    "leone_bias_span_norm": [P, ctypes.c_long, c_int, P, c_int, c_int, c_int, P, P, P, c_int, c_int, c_float, P],
+    "leone_bias_glu": [P, c_int, P, c_int, P, c_int, c_int, c_int, c_int, P],
+    "leone_add_bias": [P, P, c_int, c_int, c_int, P],
+    "leone_attention_rows_biased": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,
+                                    c_int, P, ctypes.c_long, c_int, c_int, P, c_float, c_int, P],
+    "leone_state_space_scan": [P, ctypes.c_long, c_int, c_int, c_int, c_int, P, ctypes.c_long, c_int, P, P, P, c_int, c_int, c_int,
+                               P, c_int, P, ctypes.c_long, P, ctypes.c_long, P, P, c_int, c_int, c_int, P],
     "leone_rms_mix": [P, P, c_int, c_int, c_float, c_float, P, c_int, c_int, P],
     "leone_relu_squared": [P, P, c_int, ctypes.c_long, P],
     "leone_head_gate": [P, c_int, P, ctypes.c_long, c_int, c_int, c_int, P],

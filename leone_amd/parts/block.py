@@ -16,7 +16,8 @@ class PreNormBlock(Part):
     """x1 = x + mixer(norm1(x)); x2 = x1 + feed_forward(norm2(x1)).
 
     Reference layer order: crates/leone/src/runtime.rs:9019-9050.
-    Parameters: ``norm1``, ``mixer``, ``norm2``, ``feed_forward`` (part specs).
+    Parameters: ``norm1``, ``mixer``, ``norm2``, ``feed_forward`` (part specs); the second sublayer is there
+    only if ``feed_forward`` is given.
     The residual stream is float32; each delta is added by the following norm's
     kernel, so the block returns its last delta instead of adding it.
     """
@@ -24,11 +25,13 @@ class PreNormBlock(Part):
     def __init__(self, spec: PartSpec, **context):
         self.norm1 = NORMS.build(spec["norm1"], **context)
         self.mixer = MIXERS.build(spec["mixer"], **context)
-        self.norm2 = NORMS.build(spec["norm2"], **context)
-        self.feed_forward = FEED_FORWARDS.build(spec["feed_forward"], **context)
+        self.feed_forward = FEED_FORWARDS.build(spec["feed_forward"], **context) if spec.get("feed_forward") is not None else None
+        self.norm2 = NORMS.build(spec["norm2"], **context) if spec.get("norm2") is not None else None
+        if self.feed_forward is not None and self.norm2 is None:
+            raise ValueError("a prenorm block with a feed-forward needs norm2")
 
     def parts(self):
-        return (self.norm1, self.mixer, self.norm2, self.feed_forward)
+        return tuple(part for part in (self.norm1, self.mixer, self.norm2, self.feed_forward) if part is not None)
 
     @property
     def graph_safe(self) -> bool:
@@ -48,8 +51,14 @@ class PreNormBlock(Part):
         return self.mixer.cache_need()
 
     def row_tilings(self):
-        """The tilings its parts declare (``RowTiling``)."""
-        return [part.row_tiling() for part in self.parts() if hasattr(part, "row_tiling")]
+        """The tilings its parts declare (``RowTiling``), also those of mixers inside a mixer."""
+        found = []
+        for part in self.parts():
+            if hasattr(part, "row_tiling"):
+                found.append(part.row_tiling())
+            if hasattr(part, "row_tilings"):
+                found += part.row_tilings()
+        return found
 
     prepares_next = True
 
@@ -73,6 +82,8 @@ class PreNormBlock(Part):
                      else self.mixer.forward(y, step, cache, residual=x))
         else:
             delta = self.mixer.forward(y, step, cache)
+        if self.feed_forward is None:
+            return delta
         y = self._normed(self.norm2, x, delta, step, self.feed_forward)
         if getattr(self.feed_forward, "fused_io", False):
             if next_norm is not None and getattr(self.feed_forward, "prepares_next", False):

@@ -18,7 +18,9 @@ class SwiGluMlp(Part):
     Reference: crates/leone/src/runtime.rs:9283-9319, crates/leone/src/cpu.rs:892-907.
     Parameters: ``hidden``, ``intermediate`` and tensor names ``gate``, ``up``, ``down``.
     Optional: ``activation`` (what stands on the gate instead of silu, a key of ``ops.GATE_ACTIVATIONS``),
-    ``float_output`` (what is handed back comes in float32 whatever the engine's type).
+    ``float_output`` (what is handed back comes in float32 whatever the engine's type), ``bias`` (a dict with tensor
+    names ``gate``, ``up``, ``down``: all three projections add a bias; the products then hand on float32, the biases
+    are added there, and the result comes in float32).
     """
 
     graph_safe = True
@@ -28,6 +30,10 @@ class SwiGluMlp(Part):
         self.hidden = int(p["hidden"])
         self.intermediate = int(p["intermediate"])
         self.names = {k: p[k] for k in ("gate", "up", "down")}
+        self.bias_names = dict(p["bias"]) if p.get("bias") else None
+        self.bias_in = self.bias_out = None
+        if self.bias_names:
+            self.fused_io = self.prepares_next = False      # its products hand on float32 for the biases to be added
         self.activation = str(p.get("activation") or "silu")
         if self.activation not in ops.GATE_ACTIVATIONS:
             raise ValueError(f"unknown gate activation {self.activation!r}; known: {', '.join(ops.GATE_ACTIVATIONS)}")
@@ -35,9 +41,14 @@ class SwiGluMlp(Part):
         self.w_gate_up = self.w_down = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.names["gate"], (self.intermediate, self.hidden), MATRIX),
-                TensorSpec(self.names["up"], (self.intermediate, self.hidden), MATRIX),
-                TensorSpec(self.names["down"], (self.hidden, self.intermediate), MATRIX)]
+        specs = [TensorSpec(self.names["gate"], (self.intermediate, self.hidden), MATRIX),
+                 TensorSpec(self.names["up"], (self.intermediate, self.hidden), MATRIX),
+                 TensorSpec(self.names["down"], (self.hidden, self.intermediate), MATRIX)]
+        if self.bias_names:
+            specs += [TensorSpec(self.bias_names["gate"], (self.intermediate,), VECTOR),
+                      TensorSpec(self.bias_names["up"], (self.intermediate,), VECTOR),
+                      TensorSpec(self.bias_names["down"], (self.hidden,), VECTOR)]
+        return specs
 
     fused_io = True
     prepares_next = True
@@ -48,6 +59,13 @@ class SwiGluMlp(Part):
         # multiple of 8 is filled up with zero rows; they give silu(0) * 0 = 0 and meet zero columns of
         # the down projection, so the result is unchanged.
         gate, up, down = (tensors.pop(self.names[k]) for k in ("gate", "up", "down"))
+        if self.bias_names:
+            # gate rows, then up rows: the biases are added behind the product, which therefore folds nothing in
+            self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
+            self.w_down = down.contiguous()
+            self.bias_in = torch.cat([tensors.pop(self.bias_names["gate"]), tensors.pop(self.bias_names["up"])]).contiguous()
+            self.bias_out = tensors.pop(self.bias_names["down"]).contiguous()
+            return
         pad = -self.intermediate % 8
         if pad:
             gate = torch.nn.functional.pad(gate, (0, 0, 0, pad))
@@ -62,6 +80,15 @@ class SwiGluMlp(Part):
     def forward(self, y, step: StepContext, residual: Optional[torch.Tensor] = None, next_norm=None):
         """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned),
         and with ``next_norm`` the norm that follows may come back prepared (see ``ops.linear``)."""
+        if self.bias_in is not None:
+            both = ops.linear(ops.materialize(y), self.w_gate_up, out_dtype=torch.float32)
+            if both.dim() == 3:
+                both = both.sum(dim=0)
+            activated = ops.bias_glu(both, self.bias_in, step.dtype, self.activation)
+            out = ops.linear(activated, self.w_down, out_dtype=torch.float32)
+            if out.dim() == 3:
+                out = out.sum(dim=0)
+            return ops.add_bias(out, self.bias_out)
         activated = ops.linear(y, self.w_gate_up, gated=True, activation=self.activation)
         return ops.linear(activated, self.w_down, residual=residual, next_norm=next_norm,
                           out_dtype=torch.float32 if self.float_output else None)

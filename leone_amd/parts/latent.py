@@ -71,9 +71,13 @@ class LatentAttention(Part):
     on the weighted sum of the latents), so attention runs over the latents themselves, shared by all heads.
 
     Parameters: ``hidden``, ``heads``, ``dim``, ``rot_dim``, ``vdim``, ``q_rank``, ``kv_rank``, ``scale``, ``eps``,
-    ``window``, ``position`` (name of a position part that rotates neighbouring pairs; its width may be less than
-    ``rot_dim``), tensor names ``dq``, ``dq_norm``, ``uq``, ``uk``, ``uv``, ``o`` and, unless ``shared_kv``, ``dkv`` and
-    ``dkv_norm``.  ``shared_kv``: the layer has no W_dkv and reads the cache another layer writes (its run names that
+    ``window``, ``position`` (name of a position part; its width may be less than ``rot_dim``), tensor names ``dq``,
+    ``dq_norm``, ``uq``, ``uk``, ``uv``, ``o`` and, unless ``shared_kv``, ``dkv`` and ``dkv_norm``.  With ``q_rank`` None
+    the queries come straight from the input, q = W_q y, and the tensor name ``q`` stands for ``dq``, ``dq_norm`` and
+    ``uq``.  The kernels rotate neighbouring pairs (2i, 2i + 1); a position part that pairs element i with element
+    i + R/2 is served by putting the rows of W_q's (W_uq's) rotated part and of W_dkv's last ``rot_dim`` rows in the order
+    (0, R/2, 1, R/2 + 1, ...) when the weights are bound: the rotated parts only ever meet each other in a dot product,
+    which no common reordering of its two sides changes.  ``shared_kv``: the layer has no W_dkv and reads the cache another layer writes (its run names that
     layer's cache slot and does not write).  ``retain_window``: what the cache must keep if layers with wider windows
     read it too (by default this layer's ``window``; 0: everything).
     """
@@ -82,13 +86,15 @@ class LatentAttention(Part):
 
     def __init__(self, spec: PartSpec, positions: Optional[dict] = None, **_):
         p = spec.params
-        self.hidden, self.heads, self.dim, self.rot_dim, self.vdim, self.q_rank, self.kv_rank = (
-            int(p[k]) for k in ("hidden", "heads", "dim", "rot_dim", "vdim", "q_rank", "kv_rank"))
+        self.hidden, self.heads, self.dim, self.rot_dim, self.vdim, self.kv_rank = (
+            int(p[k]) for k in ("hidden", "heads", "dim", "rot_dim", "vdim", "kv_rank"))
+        self.q_rank = int(p["q_rank"]) if p.get("q_rank") else None
         self.scale, self.eps = float(p["scale"]), float(p["eps"])
         self.window = int(p["window"]) if p.get("window") else None
         self.retain_window = self.window if "retain_window" not in p else (p["retain_window"] or None)
         self.shared_kv = bool(p.get("shared_kv", False))
-        keys = ("dq", "dq_norm", "uq", "uk", "uv", "o") + (() if self.shared_kv else ("dkv", "dkv_norm"))
+        keys = (("q",) if self.q_rank is None else ("dq", "dq_norm", "uq")) + ("uk", "uv", "o") + \
+            (() if self.shared_kv else ("dkv", "dkv_norm"))
         self.names = {k: p[k] for k in keys}
         self.position = (positions or {}).get(p.get("position")) if p.get("position") else None
         if p.get("position") and self.position is None:
@@ -100,8 +106,11 @@ class LatentAttention(Part):
 
     def tensor_specs(self) -> List[TensorSpec]:
         n = self.names
-        specs = [TensorSpec(n["dq"], (self.q_rank, self.hidden), MATRIX), TensorSpec(n["dq_norm"], (self.q_rank,), VECTOR),
-                 TensorSpec(n["uq"], (self.heads * (self.dim + self.rot_dim), self.q_rank), MATRIX)]
+        if self.q_rank is None:
+            specs = [TensorSpec(n["q"], (self.heads * (self.dim + self.rot_dim), self.hidden), MATRIX)]
+        else:
+            specs = [TensorSpec(n["dq"], (self.q_rank, self.hidden), MATRIX), TensorSpec(n["dq_norm"], (self.q_rank,), VECTOR),
+                     TensorSpec(n["uq"], (self.heads * (self.dim + self.rot_dim), self.q_rank), MATRIX)]
         if not self.shared_kv:
             specs += [TensorSpec(n["dkv"], (self.kv_rank + self.rot_dim, self.hidden), MATRIX),
                       TensorSpec(n["dkv_norm"], (self.kv_rank,), VECTOR)]
@@ -109,42 +118,71 @@ class LatentAttention(Part):
                         TensorSpec(n["uv"], (self.heads * self.vdim, self.kv_rank), MATRIX),
                         TensorSpec(n["o"], (self.hidden, self.heads * self.vdim), MATRIX)]
 
+    def _paired(self, rows: torch.Tensor, first: int) -> torch.Tensor:
+        """``rows`` with rows first .. first + R of a part that a half-split rotation turns put in the order the
+        kernels' neighbouring pairs need: (0, R/2, 1, R/2 + 1, ...)."""
+        rotation = rotation_of(self.position)
+        if rotation.pairing != "half_split" or not rotation.rotary_dim:
+            return rows
+        half = rotation.rotary_dim // 2
+        order = torch.arange(rows.shape[0], device=rows.device)
+        turned = torch.stack([torch.arange(half), torch.arange(half) + half], dim=1).reshape(-1).to(rows.device)
+        order[first:first + 2 * half] = first + turned
+        return rows.index_select(0, order)
+
+    def _paired_heads(self, rows: torch.Tensor) -> torch.Tensor:
+        """The same for the queries' projection: the rotated part of every head."""
+        size = self.dim + self.rot_dim
+        heads = [self._paired(rows[h * size:(h + 1) * size], self.dim) for h in range(self.heads)]
+        return torch.cat(heads, dim=0)
+
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         n = self.names
-        down = [tensors.pop(n["dq"])] + ([] if self.shared_kv else [tensors.pop(n["dkv"])])
-        self.w_down = torch.cat(down, dim=0).contiguous()             # one product for both down-projections
-        self.w_uq = tensors.pop(n["uq"]).contiguous()
+        rotation = rotation_of(self.position)
+        if rotation.rotary_dim > self.rot_dim:
+            raise ValueError(f"latent attention: a rotation of {rotation.rotary_dim} elements on a part of {self.rot_dim}")
+        dkv = [] if self.shared_kv else [self._paired(tensors.pop(n["dkv"]), self.kv_rank)]
+        if self.q_rank is None:
+            down = [self._paired_heads(tensors.pop(n["q"]))] + dkv
+            self.w_uq = None
+        else:
+            down = [tensors.pop(n["dq"])] + dkv
+            self.w_uq = self._paired_heads(tensors.pop(n["uq"])).contiguous()
+        self.w_down = torch.cat(down, dim=0).contiguous()             # one product for everything that reads the input
         # a product a head: [heads, inner, outer]; W_uk as stored is [heads, dim, rank] already, W_uv is turned
         self.w_uk = tensors.pop(n["uk"]).view(self.heads, self.dim, self.kv_rank).contiguous()
         self.w_uv = tensors.pop(n["uv"]).view(self.heads, self.vdim, self.kv_rank).transpose(1, 2).contiguous()
         self.w_o = tensors.pop(n["o"]).contiguous()
-        self.q_gain = tensors.pop(n["dq_norm"]).contiguous()
+        self.q_gain = tensors.pop(n["dq_norm"]).contiguous() if self.q_rank is not None else None
         self.kv_gain = self.q_gain if self.shared_kv else tensors.pop(n["dkv_norm"]).contiguous()
-        if self.q_gain.dtype != self.kv_gain.dtype:
+        if self.q_gain is not None and self.q_gain.dtype != self.kv_gain.dtype:
             self.q_gain, self.kv_gain = self.q_gain.float(), self.kv_gain.float()
 
     def streamed_weights(self) -> List[torch.Tensor]:
-        return [self.w_down, self.w_uq, self.w_o]
+        return [w for w in (self.w_down, self.w_uq, self.w_o) if w is not None]
 
     def forward(self, y: torch.Tensor, step: StepContext, cache: LatentCacheView) -> torch.Tensor:
         rotation = rotation_of(self.position)
-        if rotation.cos is not None:
-            if rotation.pairing != "adjacent":
-                raise ValueError("latent attention rotates neighbouring pairs only")
-            if step.max_position >= rotation.cos.shape[0]:
-                raise ValueError(f"position {step.max_position} is beyond the rotary table of {rotation.cos.shape[0]} positions")
+        if rotation.cos is not None and step.max_position >= rotation.cos.shape[0]:
+            raise ValueError(f"position {step.max_position} is beyond the rotary table of {rotation.cos.shape[0]} positions")
         writes = cache.writes and not self.shared_kv
         down = ops.linear(ops.materialize(y), self.w_down, out_dtype=torch.float32)
         if down.dim() == 3:
             down = down.sum(dim=0)
-        c_q = ops.latent_prepare(down, step.dtype, self.eps, q_column=0, q_rank=self.q_rank, q_gain=self.q_gain,
-                                 kv_column=self.q_rank if writes else None, rank=self.kv_rank, rot=self.rot_dim,
-                                 kv_gain=self.kv_gain, cos=rotation.cos, sin=rotation.sin, positions=step.positions,
-                                 row_entry=step.row_entry, block_table=cache.block_table, k_pool=cache.k_pool,
-                                 v_pool=cache.v_pool)
-        q = ops.linear(c_q, self.w_uq, out_dtype=torch.float32)
-        if q.dim() == 3:
-            q = q.sum(dim=0)
+        direct = self.q_rank is None
+        q_width = self.heads * (self.dim + self.rot_dim)
+        if not direct or writes:
+            c_q = ops.latent_prepare(down, step.dtype, self.eps, q_column=None if direct else 0, q_rank=self.q_rank or 0,
+                                     q_gain=self.q_gain, kv_column=(q_width if direct else self.q_rank) if writes else None,
+                                     rank=self.kv_rank, rot=self.rot_dim, kv_gain=self.kv_gain, cos=rotation.cos,
+                                     sin=rotation.sin, positions=step.positions, row_entry=step.row_entry,
+                                     block_table=cache.block_table, k_pool=cache.k_pool, v_pool=cache.v_pool)
+        if direct:
+            q = down[:, :q_width]               # the queries came out of the same product, a slice of its rows
+        else:
+            q = ops.linear(c_q, self.w_uq, out_dtype=torch.float32)
+            if q.dim() == 3:
+                q = q.sum(dim=0)
         # W_uk on the query's side; the rotated query part behind it.  The matrix-core kernel reads its queries in bfloat16.
         cores = ops.latent_cores_supported(step.dtype, self.kv_rank, self.rot_dim, cache.page_tokens)
         q = ops.head_product(q, self.w_uk, self.heads, step.dtype if cores else torch.float32, tail=self.rot_dim,

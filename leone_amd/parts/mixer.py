@@ -8,7 +8,7 @@ import torch
 
 from .. import ops
 from ..weights.loader import MATRIX, VECTOR, TensorSpec
-from .base import MIXERS, KvNeed, Part, PartSpec, RowTiling
+from .base import CONVS, MIXERS, KvNeed, Part, PartSpec, RowTiling
 from .context import KvCacheView, StepContext
 from .position import rotation_of
 
@@ -38,6 +38,14 @@ class GqaAttention(Part):
     and reads the cache another layer writes (its run names that layer's cache slot and does not write).
     ``retain_window`` / ``retain_first``: what the cache must keep if other layers with wider masks read it too
     (by default this layer's own ``window`` and ``keep_first``; ``retain_window`` 0: everything).
+    ``bias``: a dict with tensor names ``q``, ``k``, ``v`` of biases that the projections add.  ``norm_span``
+    "projection" (with ``qk_norm_eps``): q and k are each divided by their root mean square over the whole projection,
+    all heads at once, and ``q_norm`` / ``k_norm`` have the projections' sizes (default "head": every head by itself,
+    one gain for all heads).  ``conv``: a dict ``taps``, ``q``, ``k``, ``v`` (tensor names ``[channels, taps]``): q, k
+    and v each pass a short causal convolution over time directly behind the projection; the layer then also keeps a
+    request's last ``taps - 1`` projected rows.  ``distance_slopes`` (one number a query head): head h's score for a
+    key at distance d is lowered by slopes[h] * d.  ``query_factor`` = (coef, every): the queries at position p count
+    times 1 + coef * ln(floor((p + 1) / every) + 1).
     """
 
     graph_safe = True
@@ -63,8 +71,32 @@ class GqaAttention(Part):
         self.float_output = bool(p.get("float_output", False))
         if p.get("gate"):
             self.names["gate"] = p["gate"]
-        # a value size of its own or a gate: the projection carries more than q, k and v of one size
-        self.general = self.value_dim != self.head_dim or "gate" in self.names or self.shared_kv
+        self.bias_names = dict(p["bias"]) if p.get("bias") else None
+        self.norm_span = str(p.get("norm_span") or "head")
+        if self.norm_span not in ("head", "projection"):
+            raise ValueError(f"attention: norm_span {self.norm_span!r} is neither 'head' nor 'projection'")
+        self.wide_norm = self.qk_norm_eps is not None and self.norm_span == "projection"
+        self.slope_values = [float(v) for v in p["distance_slopes"]] if p.get("distance_slopes") is not None else None
+        if self.slope_values is not None and len(self.slope_values) != self.q_heads:
+            raise ValueError(f"attention: {len(self.slope_values)} distance slopes for {self.q_heads} query heads")
+        self.query_factor = (float(p["query_factor"][0]), int(p["query_factor"][1])) if p.get("query_factor") else None
+        if self.query_factor is not None and self.query_factor[1] <= 0:
+            raise ValueError(f"attention: the query factor's period must be positive, found {self.query_factor[1]}")
+        self.conv = None
+        if p.get("conv"):
+            if self.shared_kv or self.bias_names:
+                raise ValueError("attention: convolutions behind the projections go with keys of the layer's own and no biases")
+            c = p["conv"]
+            self.conv = CONVS.build(PartSpec("causal_conv", {
+                "channels": [self.q_heads * self.head_dim, self.kv_heads * self.head_dim, self.kv_heads * self.value_dim],
+                "taps": int(c["taps"]), "weights": [c["q"], c["k"], c["v"]]}))
+        if (self.bias_names or self.wide_norm) and self.shared_kv:
+            raise ValueError("attention: biases and norms over a whole projection go with keys of the layer's own")
+        # a value size of its own, a gate, or anything between the projection and the heads: the projection carries
+        # more than q, k and v of one size, or passes through kernels of its own
+        self.general = (self.value_dim != self.head_dim or "gate" in self.names or self.shared_kv or bool(self.bias_names)
+                        or self.wide_norm or self.conv is not None or self.slope_values is not None
+                        or self.query_factor is not None)
         if self.qk_norm_eps is not None:
             self.names.update(q_norm=p["q_norm"])
             if not self.shared_kv:
@@ -72,12 +104,15 @@ class GqaAttention(Part):
         self.position = (positions or {}).get(p.get("position")) if p.get("position") else None
         if p.get("position") and self.position is None:
             raise ValueError(f"attention names position part {p.get('position')!r}, which the model does not define")
-        self.w_qkv = self.w_o = self.q_gain = self.k_gain = None
+        self.w_qkv = self.w_o = self.q_gain = self.k_gain = self.bias = self.slopes = None
 
-    def cache_need(self) -> KvNeed:
-        return KvNeed(self.kv_heads, self.head_dim, self.retain_window,
+    def cache_need(self):
+        keys = KvNeed(self.kv_heads, self.head_dim, self.retain_window,
                       value_dim=self.value_dim if self.value_dim != self.head_dim else None,
                       keep_first=self.retain_first if self.retain_window else 0)
+        if self.conv is None:
+            return keys
+        return {"kv": keys, "conv": self.conv.cache_need()}
 
     def row_tiling(self) -> RowTiling:
         """The tiles of the prompt-attention kernel."""
@@ -94,9 +129,15 @@ class GqaAttention(Part):
             gates = self.q_heads * self.value_dim if self.gate_each else self.q_heads
             specs.append(TensorSpec(self.names["gate"], (gates, self.hidden), MATRIX))
         if self.qk_norm_eps is not None:
-            specs.append(TensorSpec(self.names["q_norm"], (self.head_dim,), VECTOR))
+            q_size, k_size = ((qw, kvw) if self.wide_norm else (self.head_dim, self.head_dim))
+            specs.append(TensorSpec(self.names["q_norm"], (q_size,), VECTOR))
             if not self.shared_kv:
-                specs.append(TensorSpec(self.names["k_norm"], (self.head_dim,), VECTOR))
+                specs.append(TensorSpec(self.names["k_norm"], (k_size,), VECTOR))
+        if self.bias_names:
+            specs += [TensorSpec(self.bias_names["q"], (qw,), VECTOR), TensorSpec(self.bias_names["k"], (kvw,), VECTOR),
+                      TensorSpec(self.bias_names["v"], (self.kv_heads * self.value_dim,), VECTOR)]
+        if self.conv is not None:
+            specs += self.conv.tensor_specs()
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
@@ -114,6 +155,12 @@ class GqaAttention(Part):
             self.k_gain = self.q_gain if self.shared_kv else tensors.pop(self.names["k_norm"]).contiguous()
             if self.q_gain.dtype != self.k_gain.dtype:
                 self.q_gain, self.k_gain = self.q_gain.float(), self.k_gain.float()
+        if self.bias_names:
+            self.bias = torch.cat([tensors.pop(self.bias_names[k]) for k in ("q", "k", "v")]).contiguous()
+        if self.conv is not None:
+            self.conv.bind(tensors)
+        if self.slope_values is not None:
+            self.slopes = torch.tensor(self.slope_values, dtype=torch.float32, device=self.w_o.device)
 
     def streamed_weights(self) -> List[torch.Tensor]:
         return [self.w_qkv, self.w_o]
@@ -121,7 +168,7 @@ class GqaAttention(Part):
     fused_io = True
     prepares_next = True
 
-    def forward(self, y, step: StepContext, cache: KvCacheView,
+    def forward(self, y, step: StepContext, cache,
                 residual: Optional[torch.Tensor] = None, next_norm=None):
         """``y`` may be a norm still to be done; with ``residual`` the result may be added there (None returned),
         and with ``next_norm`` the norm that follows may come back prepared (see ``ops.linear``)."""
@@ -129,9 +176,23 @@ class GqaAttention(Part):
         rotation = rotation_of(self.position)
         if rotation.cos is not None and step.max_position >= rotation.cos.shape[0]:
             raise ValueError(f"position {step.max_position} is beyond the rotary table of {rotation.cos.shape[0]} positions")
+        conv_state = None
+        if isinstance(cache, dict):
+            cache, conv_state = cache["kv"], cache.get("conv")
         if self.general:
             proj = ops.linear(y, self.w_qkv, out_dtype=torch.float32)
-            q = ops.qk_norm_rope_write(proj, self.q_heads, self.kv_heads, self.head_dim, self.q_gain, self.k_gain,
+            if proj.dim() == 3:
+                proj = proj.sum(dim=0)
+            heads = proj
+            qw, kw, vw = self.q_heads * self.head_dim, self.kv_heads * self.head_dim, self.kv_heads * self.value_dim
+            if self.conv is not None:
+                # q, k and v pass their filters side by side in one launch; the gates' columns stay where they are
+                heads = self.conv.forward(proj[:, :qw + kw + vw], step, conv_state, torch.float32)
+            if self.bias is not None or self.wide_norm:
+                spans = [(0, qw, self.q_gain), (qw, kw, self.k_gain)] if self.wide_norm else []
+                ops.bias_span_norm(heads, self.bias, spans, self.qk_norm_eps if self.wide_norm else 1.0, round_to=step.dtype)
+            head_gains = (None, None) if self.wide_norm else (self.q_gain, self.k_gain)
+            q = ops.qk_norm_rope_write(heads, self.q_heads, self.kv_heads, self.head_dim, head_gains[0], head_gains[1],
                                        self.qk_norm_eps if self.qk_norm_eps is not None else 1.0, rotation.cos, rotation.sin,
                                        step.positions, step.row_entry, cache.block_table, cache.k_pool, cache.v_pool,
                                        write_cache=cache.writes and not self.shared_kv, out_dtype=step.dtype,
@@ -179,8 +240,9 @@ class GqaAttention(Part):
                 "prompt": "flash" if ops.prefill_attention_supported(dtype, self.head_dim, page_tokens, max_blocks) else "split_kv"}
 
     def _rows_only(self) -> bool:
-        """What the matrix-core kernels are not built for: values of another size than the keys."""
-        return self.value_dim != self.head_dim
+        """What the matrix-core kernels are not built for: values of another size than the keys, scores lowered with
+        the distance, queries that grow with the position."""
+        return self.value_dim != self.head_dim or self.slope_values is not None or self.query_factor is not None
 
     def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Long prompt portions through the prompt kernel, the other rows through the split-KV kernel; the
@@ -193,7 +255,8 @@ class GqaAttention(Part):
                 not ops.decode_attention_supported(q.dtype, self.head_dim, cache.page_tokens, group, max_blocks):
             return ops.attention_rows(q, cache.k_pool, cache.v_pool, step.positions, step.row_entry,
                                       cache.block_table, self.q_heads, self.scale, window, gate=gate,
-                                      keep_first=self.keep_first, gate_each=self.gate_each)
+                                      keep_first=self.keep_first, gate_each=self.gate_each, slopes=self.slopes,
+                                      query_factor=self.query_factor)
         first = 0
         out = torch.empty_like(q)
         tiled = step.tiled.get(self.row_tiling())

@@ -15,6 +15,8 @@ class RmsNorm(Part):
     """y = (x * gain) / sqrt(mean(x^2) + eps); the gain multiplies directly (not 1 + gain).
 
     Reference: crates/leone/src/cpu.rs:1642-1663.  Parameters: ``size``, ``eps``, ``weight`` (tensor name).
+    Optional: ``weight_offset`` (a number): the stored weight lies around zero and the gain is offset + weight; the
+    sum is made once, in float32, when the weights are bound, and the kernels see an ordinary gain.
     """
 
     graph_safe = True
@@ -23,6 +25,7 @@ class RmsNorm(Part):
         self.size = int(spec["size"])
         self.eps = float(spec["eps"])
         self.weight_name = spec["weight"]
+        self.weight_offset = float(spec["weight_offset"]) if spec.get("weight_offset") is not None else None
         self.gain: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -30,6 +33,8 @@ class RmsNorm(Part):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.gain = tensors[self.weight_name].contiguous()
+        if self.weight_offset is not None:
+            self.gain = (self.gain.float() + self.weight_offset).contiguous()
 
     def add_norm(self, x: torch.Tensor, delta: Optional[torch.Tensor], out_dtype: torch.dtype,
                  rows: Optional[torch.Tensor] = None) -> torch.Tensor:

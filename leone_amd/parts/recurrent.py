@@ -286,23 +286,106 @@ class GatedMemoryMixer(Part):
         return ops.linear(y, self.w_o, out_dtype=torch.float32)
 
 
+@MIXERS.register("state_space")
+class StateSpaceMixer(Part):
+    """A selective state-space layer with one decay a head (Mamba-2).
+
+    One input projection gives, side by side, z (``heads * vdim``), x (``heads * vdim``), B and C (``groups * state``
+    each) and a step size a head.  x, B and C together pass a short causal convolution per channel (with a bias) and
+    silu.  dt = softplus(step + dt_bias); per head, with group g = head // (heads / groups):
+    S <- exp(-exp(A_log) dt) S + dt B_g x^T (S is ``state`` x ``vdim``, float32, from zero), y = S^T C_g + D x.
+    y times silu(z), then normed in ``norm_groups`` equal runs of columns, each by its own root mean square, times
+    ``norm`` (all columns' size), then the output projection.  The gate stands ahead of the norm.
+
+    Parameters: ``hidden``, ``heads``, ``vdim``, ``state``, ``groups``, ``norm_groups``, ``taps``, ``eps`` and tensor
+    names ``in``, ``conv``, ``conv_bias``, ``dt_bias``, ``A_log``, ``D``, ``norm``, ``o``.
+    """
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, **context):
+        p = spec.params
+        self.hidden, self.heads, self.vdim, self.state, self.groups, self.norm_groups = (
+            int(p[k]) for k in ("hidden", "heads", "vdim", "state", "groups", "norm_groups"))
+        self.eps = float(p["eps"])
+        _check_dim("state_space", self.state)
+        self.inner = self.heads * self.vdim
+        if self.heads % self.groups:
+            raise ValueError(f"state_space: {self.heads} heads do not share {self.groups} groups evenly")
+        if self.inner % self.norm_groups:
+            raise ValueError(f"state_space: {self.inner} columns cannot be normed in {self.norm_groups} equal runs")
+        self.names = {k: p[k] for k in ("in", "conv_bias", "dt_bias", "A_log", "D", "norm", "o")}
+        bc = self.groups * self.state
+        self.conv_width = self.inner + 2 * bc
+        self.conv = CONVS.build(PartSpec("causal_conv", {"channels": self.conv_width, "taps": int(p["taps"]),
+                                                         "weights": [p["conv"]], "activation": "silu"}), **context)
+        # the projection's columns, and x, B and C within what the convolution hands on
+        self.columns = {"z": 0, "xbc": self.inner, "dt": self.inner + self.conv_width}
+        self.scan_columns = {"x": 0, "b": self.inner, "c": self.inner + bc}
+        self.w_in = self.w_o = self.norm = self.conv_bias = self.step_bias = self.rate_log = self.skip = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        n = self.names
+        return [TensorSpec(n["in"], (self.inner + self.conv_width + self.heads, self.hidden), MATRIX),
+                TensorSpec(n["conv_bias"], (self.conv_width,), VECTOR),
+                TensorSpec(n["dt_bias"], (self.heads,), VECTOR), TensorSpec(n["A_log"], (self.heads,), VECTOR),
+                TensorSpec(n["D"], (self.heads,), VECTOR), TensorSpec(n["norm"], (self.inner,), VECTOR),
+                TensorSpec(n["o"], (self.hidden, self.inner), MATRIX)] + self.conv.tensor_specs()
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        n = self.names
+        self.w_in = tensors.pop(n["in"]).contiguous()
+        self.w_o = tensors.pop(n["o"]).contiguous()
+        self.norm = tensors.pop(n["norm"]).contiguous()
+        self.conv.bind(tensors)
+        self.conv_bias = tensors.pop(n["conv_bias"]).to(self.conv.weight.dtype).contiguous()
+        self.step_bias, self.rate_log, self.skip = (tensors.pop(n[k]).contiguous() for k in ("dt_bias", "A_log", "D"))
+        if len({self.step_bias.dtype, self.rate_log.dtype, self.skip.dtype}) > 1:
+            self.step_bias, self.rate_log, self.skip = self.step_bias.float(), self.rate_log.float(), self.skip.float()
+
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_in, self.w_o]
+
+    def cache_need(self):
+        return {"conv": self.conv.cache_need(), "memory": StateNeed((self.heads, self.state * self.vdim), torch.float32)}
+
+    def forward(self, h: torch.Tensor, step: StepContext, cache) -> torch.Tensor:
+        c = self.columns
+        proj = ops.linear(ops.materialize(h), self.w_in, out_dtype=torch.float32)
+        if proj.dim() == 3:
+            proj = proj.sum(dim=0)
+        conv_cache = cache["conv"]
+        xbc = ops.causal_conv(proj[:, c["xbc"]:c["dt"]], self.conv.weight, conv_cache.state, step, torch.float32,
+                              activation="silu", write_state=conv_cache.writes, bias=self.conv_bias)
+        memory = cache["memory"]
+        y = ops.state_space_scan(xbc, self.scan_columns, self.groups, proj[:, c["dt"]:], self.step_bias, self.rate_log,
+                                 self.skip, memory.state, step, self.heads, self.state, self.vdim, write_state=memory.writes)
+        y = ops.head_norm_gate(y, self.norm_groups, self.inner // self.norm_groups, self.eps, step.dtype, gain=self.norm,
+                               gate=proj[:, c["z"]:c["xbc"]], activation="silu", gate_first=True)
+        return ops.linear(y, self.w_o, out_dtype=torch.float32)
+
+
 @MIXERS.register("parallel")
 class ParallelMixer(Part):
     """Several mixers side by side on the same input: each result is divided by its root mean square over the
     model width and multiplied by a plain gain of its own; the mixer's result is ``scale`` times their sum (the
-    mean for ``scale`` = 1 / branches, the default).
+    mean for ``scale`` = 1 / branches, the default).  With ``weights`` (a dict name -> number) instead of ``gains``
+    nothing is normed: the result is the sum of the branches' results, each times its weight.
 
     Parameters: ``hidden``, ``eps``, ``branches`` (a dict name -> mixer spec), ``gains`` (a dict name -> tensor
-    name), ``scale`` (optional).
+    name) or ``weights``, ``scale`` (optional, with ``gains``).
     """
 
     def __init__(self, spec: PartSpec, **context):
         p = spec.params
         self.hidden, self.eps = int(p["hidden"]), float(p["eps"])
         self.branches = {name: MIXERS.build(inner, **context) for name, inner in p["branches"].items()}
-        self.gain_names = dict(p["gains"])
-        if set(self.gain_names) != set(self.branches) or not 1 <= len(self.branches) <= 4:
-            raise ValueError("parallel: one gain for each of 1 to 4 branches")
+        self.weights = {name: float(v) for name, v in p["weights"].items()} if p.get("weights") is not None else None
+        self.gain_names = dict(p.get("gains") or {})
+        if (self.weights is None) == (not self.gain_names):
+            raise ValueError("parallel: either a gain or a weight for every branch")
+        if set(self.gain_names if self.weights is None else self.weights) != set(self.branches) or not 1 <= len(self.branches) <= 4:
+            raise ValueError("parallel: one gain, or one weight, for each of 1 to 4 branches")
         self.scale = float(p.get("scale") or 1.0 / len(self.branches))
         self.gains: Dict[str, torch.Tensor] = {}
 
@@ -331,6 +414,10 @@ class ParallelMixer(Part):
         return {name: b.cache_need() for name, b in self.branches.items()}
 
     def forward(self, h: torch.Tensor, step: StepContext, cache) -> torch.Tensor:
+        h = ops.materialize(h)
         results = [b.forward(h, step, cache.get(name)) for name, b in self.branches.items()]
+        results = [r.sum(dim=0) if r.dim() == 3 else r for r in results]
         results = [r if r.dtype == torch.float32 else r.float() for r in results]
+        if self.weights is not None:
+            return ops.weighted_mix(results, [self.weights[name] for name in self.branches])
         return ops.rms_mix(results, [self.gains[name] for name in self.branches], self.eps, self.scale)
