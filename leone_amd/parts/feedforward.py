@@ -45,9 +45,10 @@ class SwiGluMlp(Part):
                  TensorSpec(self.names["up"], (self.intermediate, self.hidden), MATRIX),
                  TensorSpec(self.names["down"], (self.hidden, self.intermediate), MATRIX)]
         if self.bias_names:
-            specs += [TensorSpec(self.bias_names["gate"], (self.intermediate,), VECTOR),
-                      TensorSpec(self.bias_names["up"], (self.intermediate,), VECTOR),
-                      TensorSpec(self.bias_names["down"], (self.hidden,), VECTOR)]
+            small = ("normal", 0.0, 0.02)
+            specs += [TensorSpec(self.bias_names["gate"], (self.intermediate,), VECTOR, init=small),
+                      TensorSpec(self.bias_names["up"], (self.intermediate,), VECTOR, init=small),
+                      TensorSpec(self.bias_names["down"], (self.hidden,), VECTOR, init=small)]
         return specs
 
     fused_io = True

@@ -134,8 +134,10 @@ class GqaAttention(Part):
             if not self.shared_kv:
                 specs.append(TensorSpec(self.names["k_norm"], (k_size,), VECTOR))
         if self.bias_names:
-            specs += [TensorSpec(self.bias_names["q"], (qw,), VECTOR), TensorSpec(self.bias_names["k"], (kvw,), VECTOR),
-                      TensorSpec(self.bias_names["v"], (self.kv_heads * self.value_dim,), VECTOR)]
+            small = ("normal", 0.0, 0.02)
+            specs += [TensorSpec(self.bias_names["q"], (qw,), VECTOR, init=small),
+                      TensorSpec(self.bias_names["k"], (kvw,), VECTOR, init=small),
+                      TensorSpec(self.bias_names["v"], (self.kv_heads * self.value_dim,), VECTOR, init=small)]
         if self.conv is not None:
             specs += self.conv.tensor_specs()
         return specs

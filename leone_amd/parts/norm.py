@@ -29,6 +29,8 @@ class RmsNorm(Part):
         self.gain: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
+        if self.weight_offset is not None:      # random weights of such a norm lie around zero, so that the gain lies around the offset
+            return [TensorSpec(self.weight_name, (self.size,), VECTOR, init=("normal", 0.0, 0.02))]
         return [TensorSpec(self.weight_name, (self.size,), VECTOR)]
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:

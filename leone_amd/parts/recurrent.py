@@ -327,8 +327,10 @@ class StateSpaceMixer(Part):
     def tensor_specs(self) -> List[TensorSpec]:
         n = self.names
         return [TensorSpec(n["in"], (self.inner + self.conv_width + self.heads, self.hidden), MATRIX),
-                TensorSpec(n["conv_bias"], (self.conv_width,), VECTOR),
-                TensorSpec(n["dt_bias"], (self.heads,), VECTOR), TensorSpec(n["A_log"], (self.heads,), VECTOR),
+                TensorSpec(n["conv_bias"], (self.conv_width,), VECTOR, init=("normal", 0.0, 0.02)),
+                # step sizes around softplus(-2 .. 0) and rates exp(0 .. 1.5): memories that reach tens of tokens back
+                TensorSpec(n["dt_bias"], (self.heads,), VECTOR, init=("uniform", -2.0, 0.0)),
+                TensorSpec(n["A_log"], (self.heads,), VECTOR, init=("uniform", 0.0, 1.5)),
                 TensorSpec(n["D"], (self.heads,), VECTOR), TensorSpec(n["norm"], (self.inner,), VECTOR),
                 TensorSpec(n["o"], (self.hidden, self.inner), MATRIX)] + self.conv.tensor_specs()
 

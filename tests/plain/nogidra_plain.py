@@ -109,8 +109,11 @@ def biased_attention(h, m, w, p):
     steps = h.shape[0]
     heads, kv_heads, dim, vdim = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
     positions = list(range(steps))
-    q, k, v = (short_convolution(h @ w[p + n].T, w[p + n + ".conv"]) for n in ("q", "k", "v"))
-    q = q * query_temperature(positions, m["q_temp"])[:, None]
+    q, k, v = (h @ w[p + n].T for n in ("q", "k", "v"))
+    if m.get("conv"):
+        q, k, v = (short_convolution(u, w[p + n + ".conv"]) for u, n in ((q, "q"), (k, "k"), (v, "v")))
+    if m.get("q_temp"):
+        q = q * query_temperature(positions, m["q_temp"])[:, None]
     i, j = torch.arange(steps, dtype=F)[:, None], torch.arange(steps, dtype=F)[None, :]
     bias = torch.stack([s * (i - j) for s in distance_slopes(heads)])
     out = softmax_heads(q.view(steps, heads, dim), k.view(steps, kv_heads, dim), v.view(steps, kv_heads, vdim),

@@ -73,7 +73,7 @@ def test_unknown_architecture_is_named():
 
 
 def test_registry_takes_another_architecture():
-    assert known_architectures() == ["Fosulix", "Pamevik", "Qwen3ForCausalLM", "Zukinex"]
+    assert known_architectures() == ["Fosulix", "Nogidra", "Pamevik", "Qwen3ForCausalLM", "Zukinex"]
 
     def toy_config(raw):
         c = Qwen3Config.from_dict({**raw, "model_type": "qwen3"})
@@ -86,7 +86,7 @@ def test_registry_takes_another_architecture():
         assert c.architecture == "ToyForCausalLM"
     finally:
         unregister_architecture("ToyForCausalLM")
-    assert known_architectures() == ["Fosulix", "Pamevik", "Qwen3ForCausalLM", "Zukinex"]
+    assert known_architectures() == ["Fosulix", "Nogidra", "Pamevik", "Qwen3ForCausalLM", "Zukinex"]
 
 
 def test_model_spec_is_built_from_parts_layer_by_layer():
