@@ -417,7 +417,38 @@ def fosulix_shape(width: int, layers: int, vocab: int, context: int) -> dict:
             "embedding": {"scale": 1.0}, "canon": {"taps": 4}, "max_positions": max(4096, context + 64), "layers": listed}
 
 
-DESIGN_SHAPES = {"pamevik": pamevik_shape, "zukinex": zukinex_shape, "fosulix": fosulix_shape}
+def nogidra_shape(width: int, layers: int, vocab: int, context: int) -> dict:
+    """Nogidra at layer sizes that resemble published models of its kinds: of three layers the first latent attention
+    (heads of 128 plain and 64 rotated elements, values of 128, a key/value latent of 512), the second softmax attention
+    beside a state-space layer (heads of 128 with four query heads a key head, half a head rotated; state-space heads
+    of 64 columns over the model's width, states of 128 rows, a group of B and C to 512 columns, convolutions of 4
+    taps), the third attention with distance slopes (heads of 128, four query heads a key head, convolutions of 4 taps
+    behind q, k and v, a query factor every 1,024 positions); windows of 1,024 everywhere; the feed-forward by turns
+    dense with biases (3 x width) and 32 experts of 3/8 width of which four are chosen."""
+    heads = width // 128
+    latent = {"type": "latent_attention",
+              "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+                        "rot": {"dims": 64, "base": 500000.0}, "mask": {"size": 1024}}}
+    side = {"type": "parallel",
+            "mixer": {"left": {"heads": heads, "kv_heads": width // 512, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                               "rot": {"dims": 64, "base": 500000.0}, "mask": {"size": 1024}},
+                      "right": {"heads": width // 64, "vdim": 64, "state": 128, "groups": width // 512,
+                                "norm_groups": width // 512, "conv": 4},
+                      "left_scale": 0.6, "right_scale": 1.1}}
+    sloped = {"type": "attention",
+              "mixer": {"heads": heads, "kv_heads": width // 512, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
+                        "mask": {"size": 1024}, "q_temp": {"coef": 0.1, "every": 1024}}}
+    dense = {"kind": "dense", "ff": 3 * width}
+    routed = {"kind": "moe", "expert": {"ff": 3 * width // 8}, "router": {"experts": 32, "top": 4}}
+    order = [latent, side, sloped]
+    return {"architecture": "Nogidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+            "max_positions": max(4096, context + 64),
+            "layers": [{**order[i % 3], "mlp": routed if i % 2 else dense} for i in range(layers)]}
+
+
+DESIGN_SHAPES = {"pamevik": pamevik_shape, "zukinex": zukinex_shape, "fosulix": fosulix_shape, "nogidra": nogidra_shape}
+# The existing design whose kernels a design's own stand closest to: measured beside it, at the same sizes.
+DESIGN_NEIGHBOURS = {"nogidra": "fosulix"}
 
 
 def state_bytes_per_request(model) -> int:
@@ -474,6 +505,10 @@ def run_design(name: str, sizes: List[str], steps: int, warmup: int) -> dict:
                               intermediate_size=3 * size["width"], vocab_size=size["vocab"],
                               max_position_embeddings=max(4096, size["context"] + 64)), size)
         points[key] = {"sizes": size, name: new, "qwen3": beside}
+        neighbour = DESIGN_NEIGHBOURS.get(name)
+        if neighbour is not None:
+            points[key][neighbour] = measure(DESIGN_SHAPES[neighbour](size["width"], size["layers"], size["vocab"],
+                                                                      max(size["context"], size["prompt"])), size)
     first = points[sizes[0]]
     return {"metric": f"decode tok/s ({name} beside qwen3 at equal width, layers and vocabulary)",
             "value": first[name]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,

@@ -120,6 +120,15 @@ __device__ inline void load_projection8(const FromProjection& f, long row_width,
 // kD16 = head_dim / 16.
 // Two tiles of keys and values are held at a time (one on its way, one being worked on): up to a head size of
 // 64 that fits three waves a SIMD, up to 128 two; larger heads need all registers.
+// Scores that fall with the distance (slopes float [q_heads] or null: head h's score at distance d is lowered by
+// slopes[h] * d) and queries that count more the further on they stand (temp_every > 0: the row's scores times
+// 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)).
+struct ScoreBias {
+    const float* slopes = nullptr;
+    float temp_coef = 0.f;
+    int temp_every = 0;
+};
+
 template <int kD16, bool kFused>
 __global__ void __launch_bounds__(kDecodeThreads, kD16 <= 4 ? 3 : kD16 <= 8 ? 2 : 1)
 attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool,
@@ -127,7 +136,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
                         const int* __restrict__ row_entry, const int* __restrict__ block_table, int max_blocks,
                         float* __restrict__ part_acc, float* __restrict__ part_ml, bf16_t* __restrict__ out,
                         int q_heads, int kv_heads, int page_shift, float to_log2, int window, int splits,
-                        FromProjection from, int keep_first) {
+                        FromProjection from, int keep_first, ScoreBias bias) {
     constexpr int kD = kD16 * 16;
     constexpr int kSteps = (kD16 + 1) / 2;           // 32-element steps of the q.k product
     extern __shared__ float smem[];                   // [waves][columns][kD] accumulators, then m and l
@@ -147,6 +156,10 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
 
     const int n = positions[row] + 1;                                    // keys 0 .. n-1 exist
     const int lo = (window > 0 && n - window > 0) ? n - window : 0;      // first key in reach
+    // this lane's column is query head kvh * group + col0 + c
+    const float to_log2_row = bias.temp_every > 0
+        ? to_log2 * (1.0f + bias.temp_coef * logf(static_cast<float>(n / bias.temp_every + 1))) : to_log2;
+    const float slope_log2 = (bias.slopes && c < cols) ? bias.slopes[kvh * group + col0 + c] * 1.4426950408889634f : 0.f;
     const int* table = block_table + static_cast<long>(row_entry[row]) * max_blocks;
     const int t_begin = lo / kTileKeys, t_end = (n + kTileKeys - 1) / kTileKeys;
     // A windowed layer may keep its first keys in sight: keys below `keep` count as in reach wherever they lie.
@@ -441,7 +454,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__
         for (int j = 0; j < 8; ++j) {
             const int key = run0 + j;
             const float raw = j < 4 ? sa[j & 3] : sb[j & 3];
-            sc[j] = (full || in_reach(key)) ? raw * to_log2 : -INFINITY;
+            sc[j] = (full || in_reach(key)) ? fmaf(raw, to_log2_row, slope_log2 * static_cast<float>(key - (n - 1))) : -INFINITY;
             tile_max = fmaxf(tile_max, sc[j]);
         }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
@@ -578,7 +591,8 @@ template <int kD16>
 static void launch_decode(const void* q, const void* k_pool, const void* v_pool, const int* positions,
                           const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
                           float* part_ml, void* out, int rows, int q_heads, int kv_heads, int page_shift, float scale,
-                          int window, int splits, const FromProjection* from, int keep_first, hipStream_t stream) {
+                          int window, int splits, const FromProjection* from, int keep_first, ScoreBias bias,
+                          hipStream_t stream) {
     const int group = q_heads / kv_heads;
     dim3 grid(rows, kv_heads * ((group + 15) / 16), splits);
     const size_t smem = decode_smem_bytes(kD16 * 16, group, max_blocks);
@@ -588,21 +602,22 @@ static void launch_decode(const void* q, const void* k_pool, const void* v_pool,
             attention_decode_kernel<kD16, true><<<grid, kDecodeThreads, smem, stream>>>(
                 nullptr, static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool), positions, row_entry,
                 block_table, max_blocks, part_acc, part_ml, static_cast<bf16_t*>(out), q_heads, kv_heads, page_shift,
-                to_log2, window, splits, *from, keep_first);
+                to_log2, window, splits, *from, keep_first, bias);
             return;
         }
     }
     attention_decode_kernel<kD16, false><<<grid, kDecodeThreads, smem, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pool), static_cast<const bf16_t*>(v_pool),
         positions, row_entry, block_table, max_blocks, part_acc, part_ml, static_cast<bf16_t*>(out), q_heads, kv_heads,
-        page_shift, to_log2, window, splits, FromProjection{}, keep_first);
+        page_shift, to_log2, window, splits, FromProjection{}, keep_first, bias);
 }
 
 static int decode_checked(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
                           const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
                           float* part_ml, int rows, int q_heads, int kv_heads, int head_dim, int page_tokens,
                           float scale, int window, int splits, const FromProjection* from, int keep_first,
-                          hipStream_t stream) {
+                          hipStream_t stream, ScoreBias bias = ScoreBias{}) {
+    LEONE_REQUIRE(bias.temp_every >= 0, "attention_decode: the query factor's period %d must not be negative", bias.temp_every);
     LEONE_REQUIRE(keep_first >= 0, "attention_decode: keep_first %d must not be negative", keep_first);
     LEONE_REQUIRE((q || from) && out && k_pool && v_pool && positions && row_entry && block_table,
                   "attention_decode: null pointer");
@@ -626,7 +641,7 @@ static int decode_checked(const void* q, void* out, const void* k_pool, const vo
 #define LEONE_DECODE_CASE(N)                                                                                      \
     case N:                                                                                                       \
         launch_decode<N>(q, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml,     \
-                         out, rows, q_heads, kv_heads, page_shift, scale, window, splits, from, keep_first, stream); \
+                         out, rows, q_heads, kv_heads, page_shift, scale, window, splits, from, keep_first, bias, stream); \
         break;
     switch (head_dim / 16) {
         LEONE_DECODE_CASE(1) LEONE_DECODE_CASE(2) LEONE_DECODE_CASE(3) LEONE_DECODE_CASE(4)
@@ -669,6 +684,18 @@ extern "C" int leone_attention_decode_kept(const void* q, void* out, const void*
                                            int splits, int keep_first, hipStream_t stream) {
     return decode_checked(q, out, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml, rows,
                           q_heads, kv_heads, head_dim, page_tokens, scale, window, splits, nullptr, keep_first, stream);
+}
+
+// The same with a distance bias and a query factor that grows with the position (see ScoreBias).
+extern "C" int leone_attention_decode_biased(const void* q, void* out, const void* k_pool, const void* v_pool,
+                                             const int* positions, const int* row_entry, const int* block_table,
+                                             int max_blocks, float* part_acc, float* part_ml, int rows, int q_heads,
+                                             int kv_heads, int head_dim, int page_tokens, float scale, int window,
+                                             int splits, int keep_first, const float* slopes, float temp_coef,
+                                             int temp_every, hipStream_t stream) {
+    return decode_checked(q, out, k_pool, v_pool, positions, row_entry, block_table, max_blocks, part_acc, part_ml, rows,
+                          q_heads, kv_heads, head_dim, page_tokens, scale, window, splits, nullptr, keep_first, stream,
+                          ScoreBias{slopes, temp_coef, temp_every});
 }
 
 // The same for a step in which every row is another request, taking the fused q/k/v projection instead of

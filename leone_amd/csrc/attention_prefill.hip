@@ -72,7 +72,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ v_pool, const int* __restrict__ positions,
                          const int* __restrict__ tiles, int n_groups, const int* __restrict__ block_table,
                          int max_blocks, int q_heads, int kv_heads, int page_shift, float scale, int window,
-                         float* __restrict__ part_acc, float* __restrict__ part_ml, int splits, int keep_first) {
+                         float* __restrict__ part_acc, float* __restrict__ part_ml, int splits, int keep_first,
+                         const float* __restrict__ slopes, float temp_coef, int temp_every) {
     constexpr int kD = kD16 * 16;
     constexpr int kRuns = kD / 8;                      // 16-byte runs of one key
     constexpr int kDT = (kD + 31) / 32;                // 32-row tiles of the second product's result
@@ -160,6 +161,12 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     // The Q^T operand and the row's own position.
     const bool row_ok = j < wave_rows;
     const int row_pos = row_ok ? p0 + j : -1;                                   // -1: the row sees no key
+    // Scores that fall with the distance and queries that count more the further on they stand, both in units of the
+    // raw dot product (the scale comes later): score = dot * row_factor - (slope / scale) * (row_pos - key).
+    const bool biased = slopes != nullptr || temp_every > 0;                    // the same for the whole launch
+    const float slope_raw = slopes ? slopes[head] / scale : 0.f;
+    const float row_factor = (temp_every > 0 && row_pos >= 0)
+        ? 1.0f + temp_coef * logf(static_cast<float>((row_pos + 1) / temp_every + 1)) : 1.0f;
     bf16x8 qreg[kD16];
     {
         const bf16_t* qrow = q + (static_cast<long>(tile_row0 + (row_ok ? j : 0)) * q_heads + head) * kD;
@@ -323,6 +330,13 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             for (int v = 0; v < 16; ++v) sc[v] += sc_odd[v];
         }
         // lane (j, h): sc[v] is row j's score of key key0 + 8 h + v (v < 8) or key0 + 16 + 8 h + v - 8
+        if (biased) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int key = key0 + 8 * h + (v & 7) + 16 * (v >> 3);
+                sc[v] = fmaf(sc[v], row_factor, slope_raw * static_cast<float>(key - row_pos));
+            }
+        }
         if (!full) {                                           // the same for the whole wave
             const int p_lo = (window > 0) ? row_pos - window + 1 : 0;
 #pragma unroll
@@ -495,7 +509,8 @@ template <int kD16>
 static int launch_prefill(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
                           const int* tiles, int n_groups, const int* block_table, int max_blocks, int q_heads,
                           int kv_heads, int page_shift, float scale, int window, float* part_acc, float* part_ml,
-                          int splits, int keep_first, hipStream_t stream) {
+                          int splits, int keep_first, const float* slopes, float temp_coef, int temp_every,
+                          hipStream_t stream) {
     const size_t shared = 2 * static_cast<size_t>(stage_runs(16 * kD16)) * sizeof(uint4) + static_cast<size_t>(max_blocks) * sizeof(int);
     static size_t allowed = 48 * 1024;                 // what a kernel may use without asking
     if (shared > allowed) {
@@ -510,7 +525,7 @@ static int launch_prefill(const void* q, void* out, const void* k_pool, const vo
     attention_prefill_kernel<kD16><<<dim3(n_groups * q_heads, splits), kPrefillThreads, shared, stream>>>(
         static_cast<const bf16_t*>(q), static_cast<bf16_t*>(out), static_cast<const bf16_t*>(k_pool),
         static_cast<const bf16_t*>(v_pool), positions, tiles, n_groups, block_table, max_blocks, q_heads, kv_heads,
-        page_shift, scale, window, part_acc, part_ml, splits, keep_first);
+        page_shift, scale, window, part_acc, part_ml, splits, keep_first, slopes, temp_coef, temp_every);
     return 0;
 }
 
@@ -548,6 +563,20 @@ extern "C" int leone_attention_prefill_kept(const void* q, void* out, const void
                                             int max_blocks, int q_heads, int kv_heads, int head_dim, int page_tokens,
                                             float scale, int window, float* part_acc, float* part_ml, int splits,
                                             int keep_first, hipStream_t stream) {
+    return leone_attention_prefill_biased(q, out, k_pool, v_pool, positions, tiles, n_groups, block_table, max_blocks, q_heads,
+                                          kv_heads, head_dim, page_tokens, scale, window, part_acc, part_ml, splits, keep_first,
+                                          nullptr, 0.f, 0, stream);
+}
+
+// The same with a distance bias (slopes float [q_heads] or null: head h's score at distance d is lowered by slopes[h] * d)
+// and a query factor that grows with the position (temp_every > 0: 1 + temp_coef * ln(floor((pos + 1) / temp_every) + 1)).
+extern "C" int leone_attention_prefill_biased(const void* q, void* out, const void* k_pool, const void* v_pool,
+                                              const int* positions, const int* tiles, int n_groups, const int* block_table,
+                                              int max_blocks, int q_heads, int kv_heads, int head_dim, int page_tokens,
+                                              float scale, int window, float* part_acc, float* part_ml, int splits,
+                                              int keep_first, const float* slopes, float temp_coef, int temp_every,
+                                              hipStream_t stream) {
+    LEONE_REQUIRE(temp_every >= 0, "attention_prefill: the query factor's period %d must not be negative", temp_every);
     LEONE_REQUIRE(keep_first >= 0 && (keep_first == 0 || window == 0 || splits == 1),
                   "attention_prefill: kept first keys (%d) beside a window come with one range of keys, not %d", keep_first, splits);
     LEONE_REQUIRE(q && out && k_pool && v_pool && positions && tiles && block_table, "attention_prefill: null pointer");
@@ -573,7 +602,7 @@ extern "C" int leone_attention_prefill_kept(const void* q, void* out, const void
     case N:                                                                                                        \
         status = launch_prefill<N>(q, out, k_pool, v_pool, positions, tiles, n_groups, block_table, max_blocks,    \
                                    q_heads, kv_heads, page_shift, scale, window, part_acc, part_ml, splits,        \
-                                   keep_first, stream);                                                            \
+                                   keep_first, slopes, temp_coef, temp_every, stream);                             \
         break;
     switch (head_dim / 16) {
         LEONE_PREFILL_CASE(1) LEONE_PREFILL_CASE(2) LEONE_PREFILL_CASE(3) LEONE_PREFILL_CASE(4)

@@ -304,6 +304,17 @@ int leone_attention_rows_biased(const void* q, void* out, const void* k_pool, co
                                 int rows, int q_heads, int kv_heads, int head_dim, int v_dim, int page_tokens,
                                 float scale, int window, const float* gate, long gate_stride, int keep_first,
                                 int gate_each, const float* slopes, float temp_coef, int temp_every, hipStream_t stream);
+// The matrix-core kernels with the same distance bias and query factor as leone_attention_rows_biased.
+int leone_attention_decode_biased(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
+                                  const int* row_entry, const int* block_table, int max_blocks, float* part_acc,
+                                  float* part_ml, int rows, int q_heads, int kv_heads, int head_dim, int page_tokens,
+                                  float scale, int window, int splits, int keep_first, const float* slopes,
+                                  float temp_coef, int temp_every, hipStream_t stream);
+int leone_attention_prefill_biased(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
+                                   const int* tiles, int n_groups, const int* block_table, int max_blocks, int q_heads,
+                                   int kv_heads, int head_dim, int page_tokens, float scale, int window, float* part_acc,
+                                   float* part_ml, int splits, int keep_first, const float* slopes, float temp_coef,
+                                   int temp_every, hipStream_t stream);
 // leone_attention_decode with the keys at positions below keep_first kept in sight of a windowed layer.
 int leone_attention_decode_kept(const void* q, void* out, const void* k_pool, const void* v_pool, const int* positions,
                                 const int* row_entry, const int* block_table, int max_blocks, float* part_acc,

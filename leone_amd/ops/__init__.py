@@ -356,9 +356,11 @@ def choose_splits(rows: int, kv_heads: int, group: int, max_context: int, units:
 def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, positions: torch.Tensor,
                      row_entry: torch.Tensor, block_table: torch.Tensor, q_heads: int, scale: float,
                      window: int = 0, max_context: int = 1, splits: Optional[int] = None,
-                     out: Optional[torch.Tensor] = None, keep_first: int = 0) -> torch.Tensor:
+                     out: Optional[torch.Tensor] = None, keep_first: int = 0, slopes: Optional[torch.Tensor] = None,
+                     query_factor: Optional[tuple] = None) -> torch.Tensor:
     """Split-KV attention on the matrix cores (bfloat16).  ``max_context`` only steers the number of splits.
-    ``keep_first``: keys at positions below it stay in sight of a windowed layer."""
+    ``keep_first``: keys at positions below it stay in sight of a windowed layer.  ``slopes`` and ``query_factor``
+    as for ``attention_rows``: scores that fall with the distance, queries that count more the further on they stand."""
     rows = q.shape[0]
     pages, kv_heads, page_tokens, head_dim = cache_dims(k_pool, v_pool)
     if q.shape[1] != q_heads * head_dim:
@@ -372,12 +374,14 @@ def attention_decode(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor
     if splits > 1:
         part_acc = torch.empty((rows * q_heads * splits * head_dim,), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((rows * q_heads * splits * 2,), dtype=torch.float32, device=q.device)
-    call("leone_attention_decode_kept", _dev(q, "attention q", torch.bfloat16),
+    coef, every = query_factor if query_factor is not None else (0.0, 0)
+    call("leone_attention_decode_biased", _dev(q, "attention q", torch.bfloat16),
          _dev(out, "attention out", torch.bfloat16, q.shape), _dev(k_pool, "k pool", torch.bfloat16),
          _dev(v_pool, "v pool", torch.bfloat16), _dev(positions, "positions", torch.int32, (rows,)),
          _dev(row_entry, "row map", torch.int32, (rows,)), _dev(block_table, "block table", torch.int32),
          block_table.shape[1], _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), rows, q_heads, kv_heads,
-         head_dim, page_tokens, float(scale), int(window), int(splits), int(keep_first) if window else 0, _stream())
+         head_dim, page_tokens, float(scale), int(window), int(splits), int(keep_first) if window else 0,
+         _dev(slopes, "slopes", torch.float32, (q_heads,)), float(coef), int(every), _stream())
     return out
 
 
@@ -466,8 +470,10 @@ def choose_prefill_splits(groups: int, q_heads: int, mean_keys: int, window: int
 def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                       positions: torch.Tensor, tiles: torch.Tensor, block_table: torch.Tensor, q_heads: int,
                       scale: float, window: int = 0, mean_keys: int = 1, splits: Optional[int] = None,
-                      covered_rows: Optional[int] = None, keep_first: int = 0) -> torch.Tensor:
-    """Attention for the rows that ``tiles`` covers; writes into ``out``.
+                      covered_rows: Optional[int] = None, keep_first: int = 0, slopes: Optional[torch.Tensor] = None,
+                      query_factor: Optional[tuple] = None) -> torch.Tensor:
+    """Attention for the rows that ``tiles`` covers; writes into ``out``.  ``slopes`` and ``query_factor`` as for
+    ``attention_rows``.
 
     ``tiles`` is int32 [n, 3]: (entry, first row, rows) with at most PREFILL_TILE_ROWS consecutive rows of one
     request each, PREFILL_GROUP_TILES to a group, all tiles of a group of the same entry, unused places with
@@ -498,12 +504,14 @@ def attention_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
             raise KernelError(f"attention_prefill: {covered} covered rows of {rows}")
         part_acc = torch.empty((covered * q_heads * splits * head_dim,), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((covered * q_heads * splits * 2,), dtype=torch.float32, device=q.device)
-    call("leone_attention_prefill_kept", _dev(q, "attention q", torch.bfloat16),
+    coef, every = query_factor if query_factor is not None else (0.0, 0)
+    call("leone_attention_prefill_biased", _dev(q, "attention q", torch.bfloat16),
          _dev(out, "attention out", torch.bfloat16, q.shape), _dev(k_pool, "k pool", torch.bfloat16),
          _dev(v_pool, "v pool", torch.bfloat16), _dev(positions, "positions", torch.int32, (rows,)),
          _dev(tiles, "tiles", torch.int32), groups, _dev(block_table, "block table", torch.int32),
          block_table.shape[1], q_heads, kv_heads, head_dim, page_tokens, float(scale), int(window),
-         _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), int(splits), keep_first, _stream())
+         _dev(part_acc, "partials"), _dev(part_ml, "partial sums"), int(splits), keep_first,
+         _dev(slopes, "slopes", torch.float32, (q_heads,)), float(coef), int(every), _stream())
     return out
 
 

@@ -86,6 +86,10 @@ _PROTOTYPES = {
                                   c_int, P, ctypes.c_long, c_int, c_int, P],
     "leone_attention_decode_kept": [P, P, P, P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                     c_int, c_int, P],
+    "leone_attention_decode_biased": [P, P, P, P, P, P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                      c_int, c_int, P, c_float, c_int, P],
+    "leone_attention_prefill_biased": [P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P, P,
+                                       c_int, c_int, P, c_float, c_int, P],
     "leone_attention_prefill_kept": [P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P, P,
                                      c_int, c_int, P],
     "leone_route_topk": [P, P, c_int, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, P],

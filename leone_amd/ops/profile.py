@@ -66,6 +66,16 @@ OPERATIONS = {
     "leone_latent_attention_cores": "attention",
     "leone_residual_norm": "norm",
     "leone_depth_mix": "depth mix",
+    "leone_attention_rows_biased": "attention",
+    "leone_attention_decode_biased": "attention",
+    "leone_attention_prefill_biased": "attention",
+    "leone_causal_conv_biased": "causal conv",
+    "leone_head_norm_gate_ordered": "head norm gate",
+    "leone_weighted_mix": "branch mix",
+    "leone_state_space_scan": "state space scan",
+    "leone_bias_span_norm": "bias span norm",
+    "leone_bias_glu": "swiglu",
+    "leone_add_bias": "bias",
 }
 LIBRARY_PRODUCT = "gemm library"
 ORDER = ["embed", "norm", "gemv fused", "gemm rows", LIBRARY_PRODUCT, "gemm f32", "qknorm rope kv", "attention", "swiglu",

@@ -242,9 +242,8 @@ class GqaAttention(Part):
                 "prompt": "flash" if ops.prefill_attention_supported(dtype, self.head_dim, page_tokens, max_blocks) else "split_kv"}
 
     def _rows_only(self) -> bool:
-        """What the matrix-core kernels are not built for: values of another size than the keys, scores lowered with
-        the distance, queries that grow with the position."""
-        return self.value_dim != self.head_dim or self.slope_values is not None or self.query_factor is not None
+        """What the matrix-core kernels are not built for: values of another size than the keys."""
+        return self.value_dim != self.head_dim
 
     def _attend(self, q: torch.Tensor, step: StepContext, cache: KvCacheView, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Long prompt portions through the prompt kernel, the other rows through the split-KV kernel; the
@@ -267,12 +266,13 @@ class GqaAttention(Part):
             ops.attention_prefill(q, out, cache.k_pool, cache.v_pool, step.positions, tiled.tiles,
                                   cache.block_table, self.q_heads, self.scale, window,
                                   mean_keys=tiled.mean_keys or step.max_position + 1, covered_rows=tiled.rows,
-                                  keep_first=self.keep_first)
+                                  keep_first=self.keep_first, slopes=self.slopes, query_factor=self.query_factor)
             first = tiled.rows
         if first < step.rows:
             ops.attention_decode(q[first:], cache.k_pool, cache.v_pool, step.positions[first:],
                                  step.row_entry[first:], cache.block_table, self.q_heads, self.scale, window,
-                                 max_context=step.max_position + 1, out=out[first:], keep_first=self.keep_first)
+                                 max_context=step.max_position + 1, out=out[first:], keep_first=self.keep_first,
+                                 slopes=self.slopes, query_factor=self.query_factor)
         if gate is None:
             return out
         # a gate for every element is a gate a head of one element
