@@ -15,7 +15,11 @@
 
 namespace leone {
 
-constexpr int kSpanThreads = 256;
+// Threads a row: many for steps of few rows (a row is then a handful of trips to memory), fewer from kSpanManyRows rows
+// on, so that many rows are in flight on a compute unit.
+constexpr int kSpanThreadsFew = 1024;
+constexpr int kSpanThreadsMany = 256;
+constexpr int kSpanManyRows = 512;
 constexpr int kMaxSpans = 4;
 
 struct NormSpans {
@@ -23,6 +27,7 @@ struct NormSpans {
     AnyVec gain[kMaxSpans];
 };
 
+template <int kSpanThreads>
 __global__ void __launch_bounds__(kSpanThreads)
 bias_span_norm_kernel(float* __restrict__ rows, long stride, AnyVec bias, int biased, int round_bf16, NormSpans spans,
                       int n_spans, float eps) {
@@ -94,8 +99,12 @@ extern "C" int leone_bias_span_norm(float* rows_at, long stride, int rows, const
         spans.width[s] = widths[s];
         spans.gain[s] = AnyVec{gains[s], gain_dtype};
     }
-    bias_span_norm_kernel<<<rows, kSpanThreads, 0, stream>>>(rows_at, stride, AnyVec{bias, bias_dtype}, biased, round_bf16, spans,
-                                                             n_spans, eps);
+    if (rows >= kSpanManyRows)
+        bias_span_norm_kernel<kSpanThreadsMany><<<rows, kSpanThreadsMany, 0, stream>>>(rows_at, stride, AnyVec{bias, bias_dtype}, biased,
+                                                                                      round_bf16, spans, n_spans, eps);
+    else
+        bias_span_norm_kernel<kSpanThreadsFew><<<rows, kSpanThreadsFew, 0, stream>>>(rows_at, stride, AnyVec{bias, bias_dtype}, biased,
+                                                                                    round_bf16, spans, n_spans, eps);
     LEONE_LAUNCH_CHECK("bias_span_norm");
     return 0;
 }

@@ -81,7 +81,7 @@ __global__ void __launch_bounds__(kGsThreads) gated_scan_kernel(GatedScanArgs p,
     int col[kGsLaneCols];
 #pragma unroll
     for (int c = 0; c < kGsLaneCols; ++c)
-        col[c] = ((blockIdx.z * (kGsThreads / kWave) + tid / kWave) * kGsLaneCols + c) * per_wave + lane % per_wave;
+        col[c] = ((blockIdx.z * (blockDim.x / kWave) + tid / kWave) * kGsLaneCols + c) * per_wave + lane % per_wave;
     const int first = seg.first, n = seg.end - seg.first;
     const int ch0 = part * kGsLaneRows;
     const int shared_head = kKind == kGsStateSpace ? head / (p.heads / p.qk_heads) : head;
@@ -101,9 +101,19 @@ __global__ void __launch_bounds__(kGsThreads) gated_scan_kernel(GatedScanArgs p,
         for (int i = 0; i < kGsLaneRows; ++i) carried[i] = 1.f;
     }
 
+    __shared__ float s_dt[kGsTokens], s_decay[kGsTokens];   // the state-space form: a row's step size and decay, made once
     for (int t0 = 0; t0 < n; t0 += kGsTokens) {
         const int here = min(kGsTokens, n - t0);
-        for (int idx = tid; idx < here * dkp; idx += kGsThreads) {
+        if (kKind == kGsStateSpace) {
+            if (tid < here) {
+                const float z = p.step[static_cast<long>(first + t0 + tid) * p.step_stride + p.step_off + head] + load_any(p.step_bias, head);
+                const float dt = z > 20.f ? z : log1pf(expf(z));
+                s_dt[tid] = dt;
+                s_decay[tid] = expf(-rate * dt);
+            }
+            __syncthreads();
+        }
+        for (int idx = tid; idx < here * dkp; idx += blockDim.x) {
             const int t = idx / dkp, i = idx % dkp;
             float qv = 0.f, fv = 1.f, kv = 0.f;
             if (kKind == kGsStateSpace) {
@@ -111,10 +121,8 @@ __global__ void __launch_bounds__(kGsThreads) gated_scan_kernel(GatedScanArgs p,
                     const long r = first + t0 + t;
                     const float* base = p.proj + r * p.stride;
                     qv = base[p.q_off + shared_head * p.dim + i];
-                    const float z = p.step[r * p.step_stride + p.step_off + head] + load_any(p.step_bias, head);
-                    const float dt = z > 20.f ? z : log1pf(expf(z));
-                    fv = expf(-rate * dt);
-                    kv = p.no_input ? 0.f : dt * base[p.k_off + shared_head * p.dim + i];
+                    fv = s_decay[t];
+                    kv = p.no_input ? 0.f : s_dt[t] * base[p.k_off + shared_head * p.dim + i];
                 }
             } else if (i < p.dim) {
                 const float* base = p.proj + static_cast<long>(first + t0 + t) * p.stride;
@@ -270,11 +278,15 @@ extern "C" int leone_state_space_scan(const float* xbc, long stride, int x_off, 
                     gate_product, out, heads, dim, vdim, groups_bc, b_off, step, step_stride, step_off,
                     AnyVec{step_bias, vec_dtype}, AnyVec{rate_log, vec_dtype}, AnyVec{skip, vec_dtype}};
     const int groups = gs_lane_groups(dim);
-    const int per_block = (kGsThreads / kWave) * (kWave / groups) * kGsLaneCols;
+    // heads of few columns: a workgroup of as many waves as hold them (a wave holds 2 * 64 / groups columns), so that no
+    // wave stands idle beside the others
+    const int per_wave = (kWave / groups) * kGsLaneCols;
+    const int waves = ceil_div(vdim, per_wave) < kGsThreads / kWave ? ceil_div(vdim, per_wave) : kGsThreads / kWave;
+    const int per_block = waves * per_wave;
     const dim3 grid(n_segments, heads, ceil_div(vdim, per_block));
     const size_t shared = 3 * kGsTokens * groups * kGsLaneRows * sizeof(float);
-    if (gate_product) gated_scan_kernel<true, kGsStateSpace><<<grid, kGsThreads, shared, stream>>>(a, groups);
-    else gated_scan_kernel<false, kGsStateSpace><<<grid, kGsThreads, shared, stream>>>(a, groups);
+    if (gate_product) gated_scan_kernel<true, kGsStateSpace><<<grid, waves * kWave, shared, stream>>>(a, groups);
+    else gated_scan_kernel<false, kGsStateSpace><<<grid, waves * kWave, shared, stream>>>(a, groups);
     LEONE_LAUNCH_CHECK("state_space_scan");
     return 0;
 }
