@@ -460,3 +460,122 @@ def test_feed_forwards_and_norm_alone(dtype_name):
         want = plain.offset_norm((x + delta).to(F), wide["l0.norm1"], raw["norm"]["eps"])
         assert torch.allclose(got.double(), want, atol=1e-5, rtol=1e-5)
         assert torch.allclose(stream.cpu(), x + delta)
+
+
+def sloped_reference(q, k, v, positions, scale, window, slopes, factor, group):
+    """Plain attention of single rows: q [rows, H, d] at ``positions`` against all keys k [n, G, d], values v [n, G, e];
+    head h's score for key j is q . k * scale * factor(p) - slopes[h] * (p - j), keys j <= p within the window."""
+    out = torch.zeros(len(positions), q.shape[1], v.shape[2], dtype=F)
+    keys = torch.arange(k.shape[0])
+    for r, p in enumerate(positions):
+        see = (keys <= p) & ((p - keys < window) if window else torch.ones_like(keys, dtype=torch.bool))
+        grow = 1.0 + factor[0] * math.log((p + 1) // factor[1] + 1) if factor else 1.0
+        for head in range(q.shape[1]):
+            score = (k[:, head // group].double() @ q[r, head].double()) * scale * grow - slopes[head] * (p - keys).double()
+            out[r, head] = torch.softmax(score.masked_fill(~see, float("-inf")), dim=0) @ v[:, head // group].double()
+    return out
+
+
+@pytest.mark.parametrize("page_tokens", [16, 64])
+@pytest.mark.parametrize("window,factor", [(40, (0.5, 16)), (0, (0.25, 100)), (130, None), (64, (-0.05, 7)), (1, (1.0, 1))])
+def test_all_three_attention_kernels_with_slopes_and_a_query_factor(window, factor, page_tokens):
+    """The row kernel (float32 and bfloat16), the split-KV kernel (rows one by one, and cut into several parts) and the
+    prompt kernel (a portion of 420 rows that continues a request of 100) with a slope a head and queries that grow with
+    the position, against plain attention.  Every row's query points along one key: its own, the one before, the first,
+    one far back, the window's last and the one just outside it, keys on both sides of a page border; the slopes are
+    steep enough that the distance decides between keys that answer alike (rows whose query answers two keys at once)."""
+    from leone_amd import ops
+    from tests.test_gpu_fosulix import close
+    from tests.test_gpu_zukinex import paged, planted
+    n, first, heads, q_heads, dim = 520, 100, 2, 8, 32
+    k, v = planted(n, heads, dim, dim, 5 + window)
+    positions = list(range(first, n))
+    slopes = [2.0 ** (-8.0 * (h + 1) / q_heads) * (3.0 if h % 2 else 1.0) for h in range(q_heads)]
+    q = torch.zeros(len(positions), q_heads, dim)
+    for r, i in enumerate(positions):
+        kinds = [i, i - 1, 0, i // 2, i - window, i - window + 1, i - window - 1, 63, 64, i - 300]
+        j = min(max(kinds[r % len(kinds)] if window else kinds[r % 4], 0), i)
+        for head in range(q_heads):
+            key = k[j, head // 4].bfloat16().float()
+            other = k[max(j - 17, 0), head // 4].bfloat16().float()          # a second key that answers as loudly, further away
+            q[r, head] = (key / (key @ key) + (other / (other @ other) if r % 3 == 0 else 0.0)) * 12.0
+    slope_tensor = torch.tensor(slopes, dtype=torch.float32, device=DEV)
+    rows_at = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    entry = torch.zeros(len(positions), dtype=torch.int32, device=DEV)
+    for dtype, bound in ((torch.float32, 2e-5), (torch.bfloat16, 1.5e-2)):
+        kd, vd = k.to(dtype).float(), v.to(dtype).float()
+        want = sloped_reference(q.to(dtype).float(), kd, vd, positions, 1.0, window, slopes, factor, 4)
+        flat = sloped_reference(q.to(dtype).float(), kd, vd, positions, 1.0, window, [0.0] * q_heads, None, 4)
+        assert window == 1 or float((want - flat).abs().max()) > 0.2, "the slopes and the factor decide something here"
+        k_pool, v_pool, table = paged(k, v, page_tokens, dtype, 9)
+        flat_q = q.reshape(len(positions), -1).to(dtype).to(DEV)
+        out = ops.attention_rows(flat_q, k_pool, v_pool, rows_at, entry, table, q_heads, 1.0, window, slopes=slope_tensor,
+                                 query_factor=factor)
+        close(out.float().view(len(positions), q_heads, dim), want, bound, f"row kernel {dtype}")
+        if dtype == torch.float32:
+            continue
+        for splits in (None, 1, 3):
+            one = ops.attention_decode(flat_q, k_pool, v_pool, rows_at, entry, table, q_heads, 1.0, window, max_context=n,
+                                       splits=splits, slopes=slope_tensor, query_factor=factor)
+            close(one.float().view(len(positions), q_heads, dim), want, bound, f"split-KV kernel, splits {splits}")
+        tiles = ops.prefill_tiles([(0, 0, len(positions))]).to(DEV)
+        for splits in (None, 1, 2):
+            out = torch.full_like(flat_q, float("nan"))
+            ops.attention_prefill(flat_q, out, k_pool, v_pool, rows_at, tiles, table, q_heads, 1.0, window, mean_keys=300,
+                                  splits=splits, slopes=slope_tensor, query_factor=factor)
+            close(out.float().view(len(positions), q_heads, dim), want, bound, f"prompt kernel, splits {splits}")
+
+
+@pytest.mark.parametrize("rows", [1, 9, 600])
+def test_rowwise_kernels_of_biased_projections_against_torch(rows):
+    """``bias_span_norm``, ``bias_glu``, ``add_bias``, ``weighted_mix`` and ``head_norm_gate`` with the gate ahead of the
+    norm, each against the same few lines of torch in float32, at sizes that fill no run of 8 and in steps short and long
+    (the kernels pick their workgroup size by the number of rows)."""
+    from leone_amd import ops
+    gen = torch.Generator().manual_seed(rows)
+
+    def rand(*shape):
+        return torch.randn(*shape, generator=gen)
+    eps = 1e-5
+    # bias on the first 70 of 100 columns, two spans normed by themselves, the other columns untouched
+    x, bias, g1, g2 = rand(rows, 100), rand(70), 1 + 0.2 * rand(37), 1 + 0.2 * rand(20)
+    for round_to in (None, torch.bfloat16):
+        want = x.clone()
+        want[:, :70] += bias
+        if round_to is not None:
+            want[:, :70] = want[:, :70].to(round_to).float()
+        for (at, n, g) in ((0, 37, g1), (37, 20, g2)):
+            part = want[:, at:at + n]
+            want[:, at:at + n] = part / torch.sqrt((part * part).mean(dim=-1, keepdim=True) + eps) * g
+        got = ops.bias_span_norm(x.clone().to(DEV), bias.to(DEV), [(0, 37, g1.to(DEV)), (37, 20, g2.to(DEV))], eps, round_to=round_to)
+        assert torch.allclose(got.cpu(), want, atol=2e-5, rtol=2e-5), round_to
+    # the gated feed-forward's activation with both biases, either activation, either type out
+    both, b = rand(rows, 2 * 45), rand(2 * 45)
+    for activation, act in (("silu", torch.nn.functional.silu), ("gelu_tanh", lambda z: torch.nn.functional.gelu(z, approximate="tanh"))):
+        want = act(both[:, :45] + b[:45]) * (both[:, 45:] + b[45:])
+        got = ops.bias_glu(both.to(DEV), b.to(DEV), torch.float32, activation)
+        assert torch.allclose(got.cpu(), want, atol=2e-5, rtol=2e-5), activation
+        rounded = ops.bias_glu(both.to(DEV), b.to(DEV), torch.bfloat16, activation)
+        assert torch.equal(rounded.cpu(), got.cpu().to(torch.bfloat16)), activation
+    y, c = rand(rows, 53), rand(53)
+    assert torch.allclose(ops.add_bias(y.clone().to(DEV), c.to(DEV)).cpu(), y + c, atol=1e-6)
+    assert torch.allclose(ops.add_bias(y.clone().to(DEV), c.bfloat16().to(DEV)).cpu(), y + c.bfloat16().float(), atol=1e-6)
+    branches, weights = [rand(rows, 53) for _ in range(4)], [0.6, -1.1, 0.0, 2.5]
+    for count in (1, 2, 4):
+        want = sum(w * t for w, t in zip(weights[:count], branches[:count]))
+        got = ops.weighted_mix([t.to(DEV) for t in branches[:count]], weights[:count])
+        assert torch.allclose(got.cpu(), want, atol=1e-5), count
+    # y * silu(z), then every run of columns over its own root mean square, times a gain of all columns' size
+    for runs, size in ((3, 70), (1, 600), (5, 8)):
+        o, z, gain = rand(rows, runs * size), rand(rows, runs * size + 11), 1 + 0.2 * rand(runs * size)
+        gated = (o * torch.nn.functional.silu(z[:, :runs * size])).view(rows, runs, size)
+        want = (gated / torch.sqrt((gated * gated).mean(dim=-1, keepdim=True) + eps)).reshape(rows, -1) * gain
+        got = ops.head_norm_gate(o.to(DEV), runs, size, eps, torch.float32, gain=gain.to(DEV), gate=z.to(DEV)[:, :runs * size],
+                                 activation="silu", gate_first=True)
+        assert torch.allclose(got.cpu(), want, atol=3e-5, rtol=3e-5), (runs, size)
+        behind = ops.head_norm_gate(o.to(DEV), runs, size, eps, torch.float32, gain=gain.to(DEV), gate=z.to(DEV)[:, :runs * size],
+                                    activation="silu")
+        plain_o = o.view(rows, runs, size)
+        want = (plain_o / torch.sqrt((plain_o * plain_o).mean(dim=-1, keepdim=True) + eps)).reshape(rows, -1) * gain * \
+            torch.nn.functional.silu(z[:, :runs * size])
+        assert torch.allclose(behind.cpu(), want, atol=3e-5, rtol=3e-5), (runs, size)
