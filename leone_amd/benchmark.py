@@ -428,20 +428,20 @@ def nogidra_shape(width: int, layers: int, vocab: int, context: int) -> dict:
     heads = width // 128
     latent = {"type": "latent_attention",
               "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
-                        "rot": {"dims": 64, "base": 500000.0}, "mask": {"size": 1024}}}
+                        "rot": {"dims": 64, "base": 1000000.0}, "mask": {"size": 1024}}}
     side = {"type": "parallel",
             "mixer": {"left": {"heads": heads, "kv_heads": width // 512, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-                               "rot": {"dims": 64, "base": 500000.0}, "mask": {"size": 1024}},
+                               "rot": {"dims": 64, "base": 1000000.0}, "mask": {"size": 1024}},
                       "right": {"heads": width // 64, "vdim": 64, "state": 128, "groups": width // 512,
                                 "norm_groups": width // 512, "conv": 4},
-                      "left_scale": 0.6, "right_scale": 1.1}}
+                      "left_scale": 0.5, "right_scale": 0.5}}
     sloped = {"type": "attention",
               "mixer": {"heads": heads, "kv_heads": width // 512, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
                         "mask": {"size": 1024}, "q_temp": {"coef": 0.1, "every": 1024}}}
     dense = {"kind": "dense", "ff": 3 * width}
     routed = {"kind": "moe", "expert": {"ff": 3 * width // 8}, "router": {"experts": 32, "top": 4}}
     order = [latent, side, sloped]
-    return {"architecture": "Nogidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+    return {"architecture": "Nogidra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 50.0,
             "max_positions": max(4096, context + 64),
             "layers": [{**order[i % 3], "mlp": routed if i % 2 else dense} for i in range(layers)]}
 

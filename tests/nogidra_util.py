@@ -53,7 +53,7 @@ def layer(mixer, mlp=None):
     return {**mixer, "mlp": mlp}
 
 
-def config(width, vocab, layers, eps=1e-5, cap=30.0, max_positions=1024):
+def config(width, vocab, layers, eps=1e-5, cap=20.0, max_positions=1024):
     out = {"architecture": "Nogidra", "vocab": vocab, "width": width, "norm": {"eps": eps}, "max_positions": max_positions,
            "layers": layers}
     if cap is not None:
@@ -76,7 +76,7 @@ SMALL = {
         layer(parallel((2, 1, 24, 8, 24, 10000.0, None), (4, 12, 20, 1, 4, 5), 1.3, 0.4), dense(72)),
     ], cap=12.0),
     "B": config(96, 130, [
-        layer(parallel((6, 3, 16, 16, 16, 77.0, 16), (2, 24, 40, 2, 2, 4), 0.6, 1.1), dense(24)),
+        layer(parallel((6, 3, 16, 16, 16, 77.0, 16), (2, 24, 40, 2, 2, 4), 0.7, 1.25), dense(24)),
         layer(latent(1, 24, 16, 40, 16, base=77.0, mask=16), moe(5, 5, 8)),
         layer(attention(6, 6, 8, 16, taps=5, mask=40, q_temp=(-0.2, 3)), None),
         layer(latent(2, 32, 32, 32, 64, base=30000.0), moe(7, 3, 16)),
