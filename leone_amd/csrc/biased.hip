@@ -23,7 +23,7 @@ constexpr int kSpanManyRows = 512;
 constexpr int kMaxSpans = 4;
 
 struct NormSpans {
-    int offset[kMaxSpans], width[kMaxSpans];
+    int offset[kMaxSpans], width[kMaxSpans], count[kMaxSpans];   // count: the elements the mean is taken over
     AnyVec gain[kMaxSpans];
 };
 
@@ -46,7 +46,7 @@ bias_span_norm_kernel(float* __restrict__ rows, long stride, AnyVec bias, int bi
         const int width = spans.width[s];
         float ss = 0.f;
         for (int c = threadIdx.x; c < width; c += kSpanThreads) ss = fmaf(at[c], at[c], ss);
-        const float inv = 1.0f / sqrtf(block_sum<kSpanThreads>(ss, scratch) / static_cast<float>(width) + eps);
+        const float inv = 1.0f / sqrtf(block_sum<kSpanThreads>(ss, scratch) / static_cast<float>(spans.count[s]) + eps);
         for (int c = threadIdx.x; c < width; c += kSpanThreads) at[c] = at[c] * inv * load_any(spans.gain[s], c);
     }
 }
@@ -80,8 +80,8 @@ static int blocks_for(long n) { return static_cast<int>((n + 255) / 256 < 8192 ?
 using namespace leone;
 
 extern "C" int leone_bias_span_norm(float* rows_at, long stride, int rows, const void* bias, int bias_dtype, int biased,
-                                    int round_bf16, const int* offsets, const int* widths, const void* const* gains,
-                                    int gain_dtype, int n_spans, float eps, hipStream_t stream) {
+                                    int round_bf16, const int* offsets, const int* widths, const int* counts,
+                                    const void* const* gains, int gain_dtype, int n_spans, float eps, hipStream_t stream) {
     LEONE_REQUIRE(rows_at && rows > 0 && biased >= 0 && stride >= biased, "bias_span_norm: %d rows of %ld with %d biased columns",
                   rows, stride, biased);
     LEONE_REQUIRE(n_spans >= 0 && n_spans <= kMaxSpans && (n_spans == 0 || (offsets && widths && gains)),
@@ -97,6 +97,9 @@ extern "C" int leone_bias_span_norm(float* rows_at, long stride, int rows, const
                           "bias_span_norm: spans %d and %d overlap", t, s);
         spans.offset[s] = offsets[s];
         spans.width[s] = widths[s];
+        spans.count[s] = counts ? counts[s] : widths[s];
+        LEONE_REQUIRE(spans.count[s] > 0 && spans.count[s] <= widths[s], "bias_span_norm: span %d of %d elements cannot count %d",
+                      s, widths[s], spans.count[s]);
         spans.gain[s] = AnyVec{gains[s], gain_dtype};
     }
     if (rows >= kSpanManyRows)

@@ -227,11 +227,12 @@ int leone_head_norm_gate(const float* o, const float* dot, const float* top, con
                          int out_dtype, int rows, int heads, int vdim, hipStream_t stream);
 // Projections with biases (see biased.hip).  bias_span_norm, in place on float rows [rows, stride]: the first `biased` columns
 // get bias[c] (may be null) and, with round_bf16, bfloat16's rounding; then span s (columns offsets[s] .. + widths[s]) is
-// divided by its root mean square over the whole span and multiplied by gains[s] ([widths[s]]).  offsets, widths and gains
-// are host arrays.
+// divided by its root mean square over the whole span and multiplied by gains[s] ([widths[s]]); the mean is taken over
+// counts[s] elements (null: widths[s]; fewer where a span holds columns of zeros that do not count).  offsets, widths,
+// counts and gains are host arrays.
 int leone_bias_span_norm(float* rows_at, long stride, int rows, const void* bias, int bias_dtype, int biased, int round_bf16,
-                         const int* offsets, const int* widths, const void* const* gains, int gain_dtype, int n_spans,
-                         float eps, hipStream_t stream);
+                         const int* offsets, const int* widths, const int* counts, const void* const* gains, int gain_dtype,
+                         int n_spans, float eps, hipStream_t stream);
 // out[r, c] = act(gate_up[r, c] + bias[c]) * (gate_up[r, ffn + c] + bias[ffn + c]); act 0 silu, 1 the tanh form of gelu.
 int leone_bias_glu(const void* gate_up, int in_dtype, const void* bias, int bias_dtype, void* out, int out_dtype, int rows,
                    int ffn, int act, hipStream_t stream);

@@ -1329,9 +1329,12 @@ def bias_span_norm(rows: torch.Tensor, bias: Optional[torch.Tensor], spans, eps:
     """In place on float32 ``rows`` ``[n, width]``: the first ``len(bias)`` columns get their bias (None: none) and, with
     ``round_to`` bfloat16, that type's rounding (what a product kept in the engine's type would hold); then every span
     ``(offset, width, gain)`` is divided by its root mean square over the whole span, eps inside the root, and multiplied
-    by ``gain`` ``[width]``.  Up to four spans that do not overlap."""
+    by ``gain`` ``[width]``.  A span may name a fourth value, the number of elements its mean is taken over (a span
+    that holds columns of zeros that do not count).  Up to four spans that do not overlap."""
     n, width = rows.shape
-    spans = list(spans)
+    spans = [tuple(span) + ((span[1],) if len(span) == 3 else ()) for span in spans]
+    counts = (ctypes.c_int * max(len(spans), 1))(*[int(c) for _, _, _, c in spans])
+    spans = [span[:3] for span in spans]
     gains = [g for _, _, g in spans]
     if len({g.dtype for g in gains}) > 1:
         raise KernelError("bias_span_norm: the gains must come in one type")
@@ -1341,8 +1344,8 @@ def bias_span_norm(rows: torch.Tensor, bias: Optional[torch.Tensor], spans, eps:
     gain_ptrs = (ctypes.c_void_p * max(len(spans), 1))(*[_dev(g, "span gain", None, (int(w),)) for _, w, g in spans])
     call("leone_bias_span_norm", _dev(rows, "rows", torch.float32), width, n, _dev(bias, "bias"),
          _code(bias, "bias") if bias is not None else F32, biased, 1 if round_to == torch.bfloat16 else 0,
-         ctypes.cast(offsets, ctypes.c_void_p), ctypes.cast(widths, ctypes.c_void_p), ctypes.cast(gain_ptrs, ctypes.c_void_p),
-         _code(gains[0], "span gain") if gains else F32, len(spans), float(eps), _stream())
+         ctypes.cast(offsets, ctypes.c_void_p), ctypes.cast(widths, ctypes.c_void_p), ctypes.cast(counts, ctypes.c_void_p),
+         ctypes.cast(gain_ptrs, ctypes.c_void_p), _code(gains[0], "span gain") if gains else F32, len(spans), float(eps), _stream())
     return rows
 
 

@@ -62,7 +62,7 @@ _PROTOTYPES = {
     "leone_weighted_mix": [P, P, c_int, P, ctypes.c_long, P],
     "leone_causal_conv_biased": [P, c_int, ctypes.c_long, P, c_int, ctypes.c_long, P, P, c_int, P, c_int, P, c_int, P, P, P, c_int,
                                  c_int, c_int, c_int, c_int, c_int, P],
-    "leone_bias_span_norm": [P, ctypes.c_long, c_int, P, c_int, c_int, c_int, P, P, P, c_int, c_int, c_float, P],
+    "leone_bias_span_norm": [P, ctypes.c_long, c_int, P, c_int, c_int, c_int, P, P, P, P, c_int, c_int, c_float, P],
     "leone_bias_glu": [P, c_int, P, c_int, P, c_int, c_int, c_int, c_int, P],
     "leone_add_bias": [P, P, c_int, c_int, c_int, P],
     "leone_attention_rows_biased": [P, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float,

@@ -69,6 +69,12 @@ class GqaAttention(Part):
         self.retain_first = int(p.get("retain_first", self.keep_first) or 0)
         self.value_dim = int(p.get("value_dim") or self.head_dim)
         self.float_output = bool(p.get("float_output", False))
+        # The cache packs keys in runs of 8 elements and the kernels take values in pairs: heads of other sizes are
+        # filled up with zero rows of the projections (and zero columns of the output projection) when the weights are
+        # bound, which changes no score and no result.  ``file_*`` are the sizes the tensors have.
+        self.file_head_dim, self.file_value_dim = self.head_dim, self.value_dim
+        self.head_dim, self.value_dim = -(-self.head_dim // 8) * 8, -(-self.value_dim // 2) * 2
+        self.padded = (self.head_dim, self.value_dim) != (self.file_head_dim, self.file_value_dim)
         if p.get("gate"):
             self.names["gate"] = p["gate"]
         self.bias_names = dict(p["bias"]) if p.get("bias") else None
@@ -96,7 +102,10 @@ class GqaAttention(Part):
         # more than q, k and v of one size, or passes through kernels of its own
         self.general = (self.value_dim != self.head_dim or "gate" in self.names or self.shared_kv or bool(self.bias_names)
                         or self.wide_norm or self.conv is not None or self.slope_values is not None
-                        or self.query_factor is not None)
+                        or self.query_factor is not None or self.padded)
+        if self.padded and (self.shared_kv or self.gate_each or (self.qk_norm_eps is not None and not self.wide_norm)):
+            raise ValueError(f"attention: heads of {self.file_head_dim} and values of {self.file_value_dim} elements are filled up "
+                             f"to multiples of 8 and 2, which a norm a head, a gate an element and a borrowed cache do not allow")
         if self.qk_norm_eps is not None:
             self.names.update(q_norm=p["q_norm"])
             if not self.shared_kv:
@@ -119,17 +128,17 @@ class GqaAttention(Part):
         return RowTiling(ops.PREFILL_TILE_ROWS, ops.PREFILL_GROUP_TILES, ops.PREFILL_MIN_ROWS)
 
     def tensor_specs(self) -> List[TensorSpec]:
-        qw, kvw = self.q_heads * self.head_dim, self.kv_heads * self.head_dim
+        qw, kvw, vw = self.q_heads * self.file_head_dim, self.kv_heads * self.file_head_dim, self.kv_heads * self.file_value_dim
         specs = [TensorSpec(self.names["q"], (qw, self.hidden), MATRIX)]
         if not self.shared_kv:
             specs += [TensorSpec(self.names["k"], (kvw, self.hidden), MATRIX),
-                      TensorSpec(self.names["v"], (self.kv_heads * self.value_dim, self.hidden), MATRIX)]
-        specs.append(TensorSpec(self.names["o"], (self.hidden, self.q_heads * self.value_dim), MATRIX))
+                      TensorSpec(self.names["v"], (vw, self.hidden), MATRIX)]
+        specs.append(TensorSpec(self.names["o"], (self.hidden, self.q_heads * self.file_value_dim), MATRIX))
         if "gate" in self.names:
-            gates = self.q_heads * self.value_dim if self.gate_each else self.q_heads
+            gates = self.q_heads * self.file_value_dim if self.gate_each else self.q_heads
             specs.append(TensorSpec(self.names["gate"], (gates, self.hidden), MATRIX))
         if self.qk_norm_eps is not None:
-            q_size, k_size = ((qw, kvw) if self.wide_norm else (self.head_dim, self.head_dim))
+            q_size, k_size = ((qw, kvw) if self.wide_norm else (self.file_head_dim, self.file_head_dim))
             specs.append(TensorSpec(self.names["q_norm"], (q_size,), VECTOR))
             if not self.shared_kv:
                 specs.append(TensorSpec(self.names["k_norm"], (k_size,), VECTOR))
@@ -137,29 +146,49 @@ class GqaAttention(Part):
             small = ("normal", 0.0, 0.02)
             specs += [TensorSpec(self.bias_names["q"], (qw,), VECTOR, init=small),
                       TensorSpec(self.bias_names["k"], (kvw,), VECTOR, init=small),
-                      TensorSpec(self.bias_names["v"], (self.kv_heads * self.value_dim,), VECTOR, init=small)]
-        if self.conv is not None:
-            specs += self.conv.tensor_specs()
+                      TensorSpec(self.bias_names["v"], (vw,), VECTOR, init=small)]
+        if self.conv is not None:       # the filters as the file has them: one row a channel of the heads' own sizes
+            specs += [TensorSpec(name, (width, self.conv.taps), VECTOR) for name, width in zip(self.conv.names, (qw, kvw, vw))]
         return specs
+
+    def _filled(self, rows: torch.Tensor, heads: int, size: int, to: int) -> torch.Tensor:
+        """``rows`` ``[heads * size, ...]`` with every head's rows filled up with zero rows to ``to``."""
+        if size == to:
+            return rows
+        shaped = rows.reshape(heads, size, -1)
+        shaped = torch.nn.functional.pad(shaped, (0, 0, 0, to - size))
+        return shaped.reshape(heads * to, *rows.shape[1:])
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         # One product for q, k and v: a pure re-layout of the three matrices.
-        fused = [tensors.pop(self.names["q"])]
+        d, e = self.file_head_dim, self.file_value_dim
+        fused = [self._filled(tensors.pop(self.names["q"]), self.q_heads, d, self.head_dim)]
         if not self.shared_kv:
-            fused += [tensors.pop(self.names["k"]), tensors.pop(self.names["v"])]
+            fused += [self._filled(tensors.pop(self.names["k"]), self.kv_heads, d, self.head_dim),
+                      self._filled(tensors.pop(self.names["v"]), self.kv_heads, e, self.value_dim)]
         if "gate" in self.names:
             fused.append(tensors.pop(self.names["gate"]))      # the heads' gates ride along as further columns
         self.w_qkv = torch.cat(fused, dim=0).contiguous()
-        self.w_o = tensors.pop(self.names["o"]).contiguous()
+        w_o = tensors.pop(self.names["o"])
+        # zero columns of the output projection meet what the values' zero rows give
+        self.w_o = self._filled(w_o.t(), self.q_heads, e, self.value_dim).t().contiguous()
         if self.qk_norm_eps is not None:
             self.q_gain = tensors.pop(self.names["q_norm"]).contiguous()
             # a layer without keys of its own never normalises one; the kernels want the two gains together
             self.k_gain = self.q_gain if self.shared_kv else tensors.pop(self.names["k_norm"]).contiguous()
             if self.q_gain.dtype != self.k_gain.dtype:
                 self.q_gain, self.k_gain = self.q_gain.float(), self.k_gain.float()
+            if self.wide_norm:
+                self.q_gain = self._filled(self.q_gain, self.q_heads, d, self.head_dim).contiguous()
+                self.k_gain = self._filled(self.k_gain, self.kv_heads, d, self.head_dim).contiguous()
         if self.bias_names:
-            self.bias = torch.cat([tensors.pop(self.bias_names[k]) for k in ("q", "k", "v")]).contiguous()
+            self.bias = torch.cat([self._filled(tensors.pop(self.bias_names["q"]), self.q_heads, d, self.head_dim),
+                                   self._filled(tensors.pop(self.bias_names["k"]), self.kv_heads, d, self.head_dim),
+                                   self._filled(tensors.pop(self.bias_names["v"]), self.kv_heads, e, self.value_dim)]).contiguous()
         if self.conv is not None:
+            for name, heads, size, to in zip(self.conv.names, (self.q_heads, self.kv_heads, self.kv_heads), (d, d, e),
+                                             (self.head_dim, self.head_dim, self.value_dim)):
+                tensors[name] = self._filled(tensors[name], heads, size, to)
             self.conv.bind(tensors)
         if self.slope_values is not None:
             self.slopes = torch.tensor(self.slope_values, dtype=torch.float32, device=self.w_o.device)
@@ -191,7 +220,9 @@ class GqaAttention(Part):
                 # q, k and v pass their filters side by side in one launch; the gates' columns stay where they are
                 heads = self.conv.forward(proj[:, :qw + kw + vw], step, conv_state, torch.float32)
             if self.bias is not None or self.wide_norm:
-                spans = [(0, qw, self.q_gain), (qw, kw, self.k_gain)] if self.wide_norm else []
+                # a span's mean is taken over the elements the projection has in the file, not over what fills it up
+                spans = [(0, qw, self.q_gain, self.q_heads * self.file_head_dim),
+                         (qw, kw, self.k_gain, self.kv_heads * self.file_head_dim)] if self.wide_norm else []
                 ops.bias_span_norm(heads, self.bias, spans, self.qk_norm_eps if self.wide_norm else 1.0, round_to=step.dtype)
             head_gains = (None, None) if self.wide_norm else (self.q_gain, self.k_gain)
             q = ops.qk_norm_rope_write(heads, self.q_heads, self.kv_heads, self.head_dim, head_gains[0], head_gains[1],

@@ -78,8 +78,8 @@ def test_long_portions_of_the_state_space_walked_in_chunks(cases, monkeypatch, n
 
 
 ODD = nu.config(100, 301, [
-    nu.layer(nu.parallel((3, 3, 8, 10, 6, 300.0, 13), (5, 6, 7, 5, 5, 3), 0.9, 1.7), nu.dense(50)),
-    nu.layer(nu.attention(5, 1, 24, 6, taps=3, mask=64, q_temp=(0.3, 7)), nu.moe(12, 3, 18)),
+    nu.layer(nu.parallel((3, 3, 12, 9, 6, 300.0, 13), (5, 6, 7, 5, 5, 3), 0.9, 1.7), nu.dense(50)),
+    nu.layer(nu.attention(5, 1, 20, 7, taps=3, mask=64, q_temp=(0.3, 7)), nu.moe(12, 3, 18)),
     nu.layer(nu.latent(3, 10, 6, 10, 45, base=300.0, mask=13), nu.moe(3, 3, 7)),
     nu.layer(nu.parallel((1, 1, 40, 2, 2, 50.0, None), (1, 34, 70, 1, 2, 2), -1.0, 1.0), None),
     nu.layer(nu.latent(1, 20, 2, 4, 7, base=50.0), nu.dense(9)),
@@ -88,10 +88,10 @@ ODD = nu.config(100, 301, [
 
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
 def test_sizes_that_are_multiples_of_nothing(dtype_name):
-    """Width 100, vocabulary 301, latents of 45 and 7 elements, rotated parts of 6 and 2, values of 10, 6 and 2, states of
-    7 and 70 rows, feed-forwards of 50, 18, 9 and 7, a prompt of 300 tokens (the state-space layers' long portions in
+    """Width 100, vocabulary 301, latents of 45 and 7 elements, rotated parts of 6 and 2, keys of 12 and 20 elements and
+    values of 9 and 7 (heads that are filled up with zeros to what the cache packs), states of 7 and 70 rows, feed-forwards of 50, 18, 9 and 7, a prompt of 300 tokens (the state-space layers' long portions in
     chunks), pages of 64 tokens: every kernel's path for sizes that fill no run of 8 or 16."""
-    weights = nu.make_weights(ODD, 3, DTYPES[dtype_name], sharpen=1.5 if dtype_name == "float32" else 1.0)
+    weights = nu.make_weights(ODD, 3, DTYPES[dtype_name])
     gen = np.random.default_rng(1)
     requests = {f"r{i}": gen.integers(0, ODD["vocab"], size=n).tolist() for i, n in enumerate([300, 70, 5, 129])}
     expected = {rid: plain.forward(ODD, widened(weights), toks).numpy() for rid, toks in requests.items()}
@@ -285,12 +285,12 @@ def check_in_cuts(mixer, want_of, width, dtype_name, page_tokens, bound=None, ro
 
 BIASED = [nu.attention(4, 2, 16, 24, taps=3, mask=19, q_temp=(0.7, 8)), nu.attention(1, 1, 40, 8, taps=2, mask=None, q_temp=(2.0, 1)),
           nu.attention(6, 6, 8, 8, taps=5, mask=1, q_temp=None), nu.attention(8, 2, 64, 64, taps=4, mask=32, q_temp=(0.5, 30)),
-          nu.attention(3, 1, 16, 16, taps=None, mask=33, q_temp=(-0.1, 5))]
+          nu.attention(3, 1, 16, 16, taps=None, mask=33, q_temp=(-0.1, 5)), nu.attention(4, 2, 20, 7, taps=3, mask=19, q_temp=(0.7, 8))]
 
 
 @pytest.mark.parametrize("page_tokens", [16, 32])
 @pytest.mark.parametrize("dtype_name", list(DTYPES))
-@pytest.mark.parametrize("entry", BIASED, ids=lambda e: f"{e['mixer']['heads']}x{e['mixer']['dim']}")
+@pytest.mark.parametrize("entry", BIASED, ids=lambda e: f"{e['mixer']['heads']}x{e['mixer']['dim']}x{e['mixer']['vdim']}")
 def test_attention_with_slopes_alone_in_cuts_of_every_size(entry, dtype_name, page_tokens):
     """Two sequences side by side, fed in steps of 0 to 40 rows each, state slots and pages interleaved and filled with
     NaN beforehand: the convolutions' first rows see zeros, every later step the rows the step before left; a window of
@@ -325,7 +325,8 @@ SIDES = [nu.parallel((4, 2, 16, 16, 8, 100.0, 33), (3, 8, 12, 3, 1, 2), 0.8, -0.
          nu.parallel((2, 1, 24, 8, 24, 10000.0, None), (4, 12, 20, 1, 4, 5), 1.3, 0.4),
          nu.parallel((6, 3, 16, 16, 16, 77.0, 16), (2, 24, 40, 2, 2, 4), 0.0, 1.0),
          nu.parallel((8, 1, 32, 32, 16, 1000.0, 24), (8, 16, 64, 4, 2, 4), 1.0, 0.0),
-         nu.parallel((1, 1, 48, 48, 2, 20.0, 1), (1, 130, 200, 1, 1, 3), 0.5, 0.5)]
+         nu.parallel((1, 1, 48, 48, 2, 20.0, 1), (1, 130, 200, 1, 1, 3), 0.5, 0.5),
+         nu.parallel((4, 2, 12, 5, 4, 100.0, 9), (2, 6, 10, 2, 1, 2), 1.0, 0.0)]
 
 
 @pytest.mark.parametrize("page_tokens", [16, 32])
