@@ -65,7 +65,8 @@ def test_a_serving_scenario_with_one_layer(name):
 
 
 @pytest.mark.parametrize("design,operations", [("pamevik", {"outer scan", "delta scan", "layer norm"}),
-                                               ("zukinex", {"router", "experts", "attention", "norm"})])
+                                               ("zukinex", {"router", "experts", "attention", "norm"}),
+                                               ("nogidra", {"state space scan", "bias span norm", "attention", "experts"})])
 def test_another_design_beside_its_closest_relative(capsys, design, operations):
     """``--design NAME``: one line with the design's decode and prompt figures and Qwen3's at equal width, depth
     and vocabulary beside them, each with a per-operation table; the headline workload is not run."""
@@ -76,7 +77,9 @@ def test_another_design_beside_its_closest_relative(capsys, design, operations):
     record = json.loads(lines[0])
     assert record["n_gpus"] == 1 and record["steps"] == 4 and record["config"] == {"model": design, "sizes": ["w512"]}
     point = record["points"]["w512"]
-    for name in (design, "qwen3"):
+    neighbour = benchmark.DESIGN_NEIGHBOURS.get(design)       # a design with a closer relative than Qwen3 has it beside it too
+    assert (neighbour in point) == (neighbour is not None)
+    for name in (design, "qwen3") + ((neighbour,) if neighbour else ()):
         side = point[name]
         assert side["decode_tok_s"] > 0 and side["prefill_tok_s"] > 0 and side["decode_gb_per_step"] > 0
         assert abs(side["decode_tok_s"] - 2 / side["decode_ms_per_step"] * 1e3) / side["decode_tok_s"] < 1e-2
