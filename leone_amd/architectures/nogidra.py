@@ -93,18 +93,20 @@ def _feed_forward(config: NogidraConfig, i: int):
 
 def nogidra_model_spec(config: NogidraConfig) -> ModelSpec:
     positions: dict = {}
-    layers = []
+    layers, unused = [], []
     for i in range(len(config.layers)):
         p = f"l{i}."
         params = {"norm1": _norm(config, p + "norm1"), "mixer": _mixer(config, i, positions)}
         feed_forward = _feed_forward(config, i)
         if feed_forward is not None:
             params.update(norm2=_norm(config, p + "norm2"), feed_forward=feed_forward)
+        else:
+            unused.append(p + "norm2")          # a file may hold the second norm of a layer that has no second sublayer
         layers.append(PartSpec("prenorm", params))
     return ModelSpec(hidden_size=config.width, vocab_size=config.vocab, max_positions=config.max_positions,
                      embedding="embed", layers=layers, schedule=default_schedule(len(layers)),
                      final_norm=_norm(config, "final.norm"), head="head", positions=positions,
-                     logit_cap=config.logit_softcap)
+                     logit_cap=config.logit_softcap, ignore_tensors=tuple(unused))
 
 
 register_architecture(NogidraConfig.ARCHITECTURE, NogidraConfig.from_dict, nogidra_model_spec)

@@ -11,7 +11,8 @@ config.json keys: ``architecture`` ("Nogidra"), ``vocab``, ``width``, ``norm.eps
   ``parallel``          ``mixer`` = {left: {heads, kv_heads, dim, vdim, scale, rot: {dims, base}, mask: {size}},
                                      right: {heads, vdim, state, groups, norm_groups, conv}, left_scale, right_scale}
 
-``mask`` may be absent (every earlier key is seen), and so may ``conv`` and ``q_temp`` of an ``attention`` mixer.
+``mask`` may be absent (every earlier key is seen), and so may ``conv`` and ``q_temp`` of an ``attention`` mixer,
+``kv_heads`` (as many as ``heads``), ``vdim`` (``dim``) and ``scale`` (one over the root of a key's size).
 ``mlp`` is null, {kind: "dense", ff} or {kind: "moe", expert: {ff}, router: {experts, top}}.  ``max_positions``
 (optional) bounds the rotary tables and a request's length.
 """
@@ -156,8 +157,9 @@ def _biased_attention(raw: Mapping[str, Any], where: str) -> BiasedAttentionConf
     m = _sub(raw, "mixer", where)
     w = where + "mixer."
     try:
-        heads, kv_heads, dim, vdim = (m.positive_int(k) for k in ("heads", "kv_heads", "dim", "vdim"))
-        scale = m.positive_float("scale")
+        heads, dim = m.positive_int("heads"), m.positive_int("dim")
+        kv_heads, vdim = m.positive_int("kv_heads", heads), m.positive_int("vdim", dim)
+        scale = m.positive_float("scale", dim ** -0.5)
         taps = m.positive_int("conv", None)
         coef = every = None
         temp = _sub(m.raw, "q_temp", w, optional=True)
@@ -180,7 +182,7 @@ def _latent(raw: Mapping[str, Any], where: str) -> LatentAttentionConfig:
     w = where + "mixer."
     try:
         heads, dim, rot_dim, vdim, kv_rank = (m.positive_int(k) for k in ("heads", "dim", "rot_dim", "vdim", "kv_rank"))
-        scale = m.positive_float("scale")
+        scale = m.positive_float("scale", (dim + rot_dim) ** -0.5)
         rot_dims, rot_base = _rotation(m, w, rot_dim)
         window = _window(m, w)
     except ConfigError as error:
@@ -194,8 +196,9 @@ def _parallel(raw: Mapping[str, Any], where: str) -> ParallelConfig:
     try:
         left, right = _sub(m.raw, "left", w), _sub(m.raw, "right", w)
         try:
-            heads, kv_heads, dim, vdim = (left.positive_int(k) for k in ("heads", "kv_heads", "dim", "vdim"))
-            scale = left.positive_float("scale")
+            heads, dim = left.positive_int("heads"), left.positive_int("dim")
+            kv_heads, vdim = left.positive_int("kv_heads", heads), left.positive_int("vdim", dim)
+            scale = left.positive_float("scale", dim ** -0.5)
             rot_dims, rot_base = _rotation(left, w + "left.", dim)
             window = _window(left, w + "left.")
             _grouped(heads, kv_heads, w + "left.")

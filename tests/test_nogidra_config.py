@@ -63,6 +63,13 @@ def test_defaults_where_the_configuration_is_silent():
     plain_attention = config_from_dict(nu.SMALL["A"]).layers[3].mixer
     assert isinstance(plain_attention, BiasedAttentionConfig)
     assert plain_attention.taps is None and plain_attention.temp_every is None and plain_attention.window is None
+    bare = copy.deepcopy(nu.SMALL["A"])
+    for key in ("kv_heads", "vdim", "scale"):
+        del bare["layers"][0]["mixer"][key]
+    first = config_from_dict(bare).layers[0].mixer
+    assert (first.kv_heads, first.vdim, first.scale) == (4, 16, 0.25)       # as many as heads, the keys' size, 16 ** -0.5
+    # a file may hold the second norm of a layer without a feed-forward; nothing else goes unused
+    assert model_spec_for(config_from_dict(nu.SMALL["A"])).ignore_tensors == ("l2.norm2",)
 
 
 BROKEN = [
@@ -70,7 +77,8 @@ BROKEN = [
     (lambda r: r["norm"].pop("eps"), "eps"),
     (lambda r: r.update(logit_softcap=-1.0), "logit_softcap"),
     (lambda r: r["layers"][0].update(type="hgrn2"), "layers[0].type"),
-    (lambda r: r["layers"][0]["mixer"].pop("vdim"), "layers[0].mixer.vdim"),
+    (lambda r: r["layers"][0]["mixer"].pop("dim"), "layers[0].mixer.dim"),
+    (lambda r: r["layers"][0]["mixer"].update(vdim=0), "layers[0].mixer.vdim"),
     (lambda r: r["layers"][0]["mixer"].update(kv_heads=3), "layers[0].mixer.kv_heads"),
     (lambda r: r["layers"][0]["mixer"].update(conv=1), "layers[0].mixer.conv"),
     (lambda r: r["layers"][0]["mixer"]["q_temp"].update(every=0), "layers[0].mixer.q_temp.every"),
